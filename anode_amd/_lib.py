@@ -1,0 +1,103 @@
+"""ctypes loader for libanode_routines_gpu.so.
+
+The prototypes are read from include/anode_routines_gpu.h, so what Python
+calls is exactly what the C header declares (the reference's routines_gpu/lib.h
+ABI plus the additive entry points).  There is no fallback: if the shared
+library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+from typing import Dict, List, Tuple
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+REPO_ROOT = os.path.dirname(_HERE)
+HEADER_PATH = os.path.join(REPO_ROOT, "include", "anode_routines_gpu.h")
+LIBRARY_PATH = os.path.join(_HERE, "libanode_routines_gpu.so")
+STATIC_LIBRARY_PATH = os.path.join(_HERE, "libanode_routines_gpu.a")
+
+
+class KernelConfig(ctypes.Structure):
+    """Launch hints; layout fixed by the reference (routines_gpu/common.cuh:65-66)."""
+
+    _fields_ = [("block_sz", ctypes.c_uint32), ("max_block_ct", ctypes.c_uint32)]
+
+
+_SCALARS = {
+    "uint32_t": ctypes.c_uint32,
+    "int": ctypes.c_int,
+    "float": ctypes.c_float,
+    "void": None,
+}
+
+_DECL = re.compile(r"^\s*(void|int|uint32_t)\s+(anode_gpu_\w+)\s*\(([^;]*)\)\s*;", re.M)
+
+
+def _ctype_of(param: str):
+    param = param.strip()
+    if param in ("void", ""):
+        return None
+    if "*" in param:
+        return ctypes.c_void_p
+    base = param.split()[0]
+    if base == "const":
+        base = param.split()[1]
+    return _SCALARS[base]
+
+
+def parse_header(path: str = HEADER_PATH) -> Dict[str, Tuple[object, List[object], List[str]]]:
+    """name -> (restype, argtypes, parameter names) for every entry point declared in the header."""
+    text = open(path, "r").read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = text.replace("ANODE_LAUNCH_TAIL", "const struct KernelConfig *cfg, struct CUstream_st *stream")
+    out = {}
+    for ret, name, params in _DECL.findall(text):
+        argtypes, names = [], []
+        for p in params.split(","):
+            t = _ctype_of(p)
+            if t is None:
+                continue
+            argtypes.append(t)
+            names.append(p.replace("*", " ").split()[-1])
+        out[name] = (_SCALARS[ret], argtypes, names)
+    return out
+
+
+class Library:
+    """The loaded shared library with typed entry points."""
+
+    def __init__(self, path: str = LIBRARY_PATH):
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                f"{path} is missing: build it with `make -C anode_amd/csrc` "
+                "(or __graft_entry__.build()); there is no fallback implementation"
+            )
+        self.path = path
+        self.cdll = ctypes.CDLL(path)
+        self.prototypes = parse_header()
+        for name, (restype, argtypes, _) in self.prototypes.items():
+            fn = getattr(self.cdll, name)  # AttributeError if the header and the library disagree
+            fn.restype = restype
+            fn.argtypes = argtypes
+        # not in the public header: host-side probes and tuning knobs
+        self.cdll.anode_gpu_plan_reduce.restype = None
+        self.cdll.anode_gpu_plan_reduce.argtypes = [ctypes.c_uint32] * 3 + [ctypes.c_int, ctypes.c_void_p]
+        self.cdll.anode_gpu_fastdiv_probe.restype = ctypes.c_uint32
+        self.cdll.anode_gpu_fastdiv_probe.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+        self.cdll.anode_gpu_set_tuning.restype = ctypes.c_int
+        self.cdll.anode_gpu_set_tuning.argtypes = [ctypes.c_int, ctypes.c_int]
+
+    def symbol(self, name: str):
+        return getattr(self.cdll, name)
+
+
+_LIB = None
+
+
+def load() -> Library:
+    global _LIB
+    if _LIB is None:
+        _LIB = Library()
+    return _LIB

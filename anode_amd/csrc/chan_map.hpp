@@ -1,0 +1,127 @@
+// Elementwise maps over a packed [S, C, N] array (S fastest) whose arithmetic
+// depends on the element's channel c: out[s,c,n] = f(param[c], a[s,c,n], b[s,c,n]).
+//
+// The array is walked as a flat sequence of 16-byte groups, exactly like the
+// channel-free maps; the channel of a group's first element comes from two
+// multiply-high divisions by launch-invariant divisors (no hardware divide per
+// element), and the (s, c) pair is then advanced incrementally inside the
+// group, reloading the per-channel parameters only when a channel boundary is
+// crossed.  This keeps full 16-byte accesses for every S, including S that is
+// not a multiple of 4 (7x7 feature maps) and S == 1.
+#pragma once
+
+#include "common.hpp"
+
+namespace anode {
+
+// Op concept:
+//   struct Param;                                  per-channel values
+//   __device__ Param load(uint32_t c) const;
+//   __device__ float value(const Param&, float a, float b, uint32_t s) const;
+//   __device__ float accum(const Param&, float a, float b, uint32_t s, float old) const;
+// where s is the element's position inside its channel run.
+template <typename V> struct VecLanes;
+template <> struct VecLanes<float> { static constexpr int n = 1; };
+template <> struct VecLanes<f32x4> { static constexpr int n = 4; };
+
+template <typename V>
+__device__ inline float lane_get(const V &v, int k);
+template <>
+__device__ inline float lane_get<float>(const float &v, int) { return v; }
+template <>
+__device__ inline float lane_get<f32x4>(const f32x4 &v, int k) { return v[k]; }
+
+template <typename V>
+__device__ inline void lane_set(V &v, int k, float x);
+template <>
+__device__ inline void lane_set<float>(float &v, int, float x) { v = x; }
+template <>
+__device__ inline void lane_set<f32x4>(f32x4 &v, int k, float x) { v[k] = x; }
+
+template <typename V, int NIN, bool ACC, int UNROLL, typename Op>
+__global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
+                                                          FastDiv div_c, Op op, const float *a_,
+                                                          const float *b_, float *out_, int nontemporal) {
+  constexpr int L = VecLanes<V>::n;
+  const V *a = reinterpret_cast<const V *>(a_);
+  const V *b = reinterpret_cast<const V *>(b_);
+  V *out = reinterpret_cast<V *>(out_);
+  const uint32_t S = div_s.d, C = div_c.d;
+  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
+  const uint32_t stride = gridDim.x * kTile;
+  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+    V va[UNROLL], vb[UNROLL], vo[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) {
+        if (NIN >= 1) va[u] = a[g];
+        if (NIN >= 2) vb[u] = b[g];
+        if (ACC) vo[u] = out[g];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) {
+        uint32_t q, s;
+        div_s.divmod(g * uint32_t(L), q, s);
+        uint32_t c = q - div_c.div(q) * C;
+        typename Op::Param p = op.load(c);
+        V r;
+#pragma unroll
+        for (int k = 0; k < L; ++k) {
+          const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
+          const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
+          const float v = ACC ? op.accum(p, x, y, s, lane_get<V>(vo[u], k)) : op.value(p, x, y, s);
+          lane_set<V>(r, k, v);
+          if (k + 1 < L) {
+            if (++s == S) {
+              s = 0;
+              c = (c + 1 == C) ? 0 : c + 1;
+              p = op.load(c);
+            }
+          }
+        }
+        if (nontemporal) {
+          __builtin_nontemporal_store(r, &out[g]);
+        } else {
+          out[g] = r;
+        }
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * uint32_t(L) + threadIdx.x;
+    uint32_t q, s;
+    div_s.divmod(i, q, s);
+    const uint32_t c = q - div_c.div(q) * C;
+    const typename Op::Param p = op.load(c);
+    const float x = (NIN >= 1) ? a_[i] : 0.0f;
+    const float y = (NIN >= 2) ? b_[i] : 0.0f;
+    out_[i] = ACC ? op.accum(p, x, y, s, out_[i]) : op.value(p, x, y, s);
+  }
+}
+
+// a, b may be null when NIN says they are unused.
+template <int NIN, bool ACC, typename Op>
+void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
+                     const float *b, float *out, CUstream_st *stream) {
+  const uint32_t len = checked_len(S, C, N, symbol);
+  if (len == 0) return;
+  const Tuning &t = tuning();
+  hipStream_t s = as_stream(stream);
+  const FastDiv div_s(S), div_c(C);
+  const bool vec = aligned16(out) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
+  if (vec) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    chan_map_kernel<f32x4, NIN, ACC, 4, Op>
+        <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, t.nontemporal);
+  } else {
+    chan_map_kernel<float, NIN, ACC, 4, Op>
+        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, out, 0);
+  }
+  note_launch(symbol);
+}
+
+}  // namespace anode

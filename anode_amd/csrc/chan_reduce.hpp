@@ -1,0 +1,295 @@
+// Per-channel reductions over a packed [S, C, N] array (S fastest):
+//   out[c] = finalize(c, sum_{s,n} term0(a, b), sum_{s,n} term1(a, b)).
+//
+// One channel of a batch is N separate runs of S contiguous floats, and the
+// number of channels is often far smaller than the number of compute units, so
+// the work is cut into tiles that are independent of C:
+//
+//   "chunk" tiles (S large): SB contiguous positions of one (n, c) run, for NB
+//     consecutive samples.  Every element of the tile belongs to one channel;
+//     threads stream 16-byte groups and keep a few fp64 running sums.
+//   "whole" tiles (S <= 4096): CB whole channels that are adjacent in memory
+//     (CB*S contiguous floats), for NB consecutive samples.  A thread owns
+//     fixed positions of that span and adds the same positions of every sample
+//     into per-position fp64 sums, so accesses stay contiguous and 16-byte wide
+//     even when S is odd; at the end of the tile the positions are folded to
+//     channels through LDS.
+//
+// Each tile leaves one fp64 partial per (channel, tile) in a scratch buffer
+// and a second, tiny kernel adds a channel's partials in a fixed order and
+// applies the operator's finalisation.  All sums are fp64 and every order of
+// addition is fixed by the launch geometry, so results are reproducible from
+// run to run and independent of scheduling.  When a channel has a single
+// partial the first kernel finalises directly.
+#pragma once
+
+#include "chan_map.hpp"
+#include "common.hpp"
+
+namespace anode {
+
+constexpr uint32_t kTilePos = 4096;   // positions of a "whole" tile: 32 KiB of fp64 in LDS
+constexpr uint32_t kMaxTileChans = 256;
+
+struct ReducePlan {
+  uint32_t S, C, N;
+  uint32_t whole;     // 1: whole-channel tiles, 0: chunk tiles
+  uint32_t CB;        // channels per tile (whole)
+  uint32_t SB;        // positions per tile (chunk)
+  uint32_t n_ctiles;  // whole: ceil(C / CB); chunk: C
+  uint32_t n_stiles;  // whole: 1; chunk: ceil(S / SB)
+  uint32_t NB;        // samples per tile
+  uint32_t n_ntiles;  // ceil(N / NB)
+  uint32_t ppc;       // partials per channel = n_stiles * n_ntiles
+  uint32_t vec;       // 1: 16-byte accesses are legal for this geometry
+  uint32_t grid;      // n_ctiles * n_stiles * n_ntiles
+};
+
+// Host-side tiling decision; `ptrs_aligned` says whether every element array
+// is 16-byte aligned.  Exposed (anode_gpu_plan_reduce) so that it can be
+// checked without a device.
+ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target);
+
+#if defined(__HIPCC__)
+
+// Op concept:
+//   static constexpr int NIN  (1 or 2 element inputs), NACC (1 or 2 sums);
+//   struct Param;  __device__ Param load(uint32_t c) const;
+//   __device__ void term(const Param&, float a, float b, double &s0, double &s1) const;
+//   __device__ void finalize(uint32_t c, double s0, double s1) const;   // writes the output(s)
+
+template <typename Op, typename V>
+__global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl, Op op,
+                                                                   const float *__restrict__ a,
+                                                                   const float *__restrict__ b,
+                                                                   double *__restrict__ part) {
+  constexpr int W = VecLanes<V>::n;
+  constexpr int U = 4;
+  __shared__ double lds[kBlock / kWave];
+
+  const uint32_t st = blockIdx.x % pl.n_stiles;
+  const uint32_t r = blockIdx.x / pl.n_stiles;
+  const uint32_t c = r % pl.C;
+  const uint32_t nt = r / pl.C;
+  const uint32_t s0 = st * pl.SB;
+  const uint32_t sl = min(pl.SB, pl.S - s0);
+  const uint32_t LG = sl / uint32_t(W);
+  const uint32_t n0 = nt * pl.NB;
+  const uint32_t n1 = min(pl.N, n0 + pl.NB);
+  const typename Op::Param prm = op.load(c);
+
+  double acc0[U], acc1[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) acc0[u] = acc1[u] = 0.0;
+
+  for (uint32_t n = n0; n < n1; ++n) {
+    const size_t row = (size_t(n) * pl.C + c) * pl.S + s0;
+    const V *pa = reinterpret_cast<const V *>(a + row);
+    const V *pb = reinterpret_cast<const V *>(b + row);
+    for (uint32_t jb = 0; jb < LG; jb += uint32_t(U) * kBlock) {
+      V va[U], vb[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
+        if (j < LG) {
+          va[u] = pa[j];
+          if (Op::NIN >= 2) vb[u] = pb[j];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
+        if (j < LG) {
+#pragma unroll
+          for (int k = 0; k < W; ++k) {
+            op.term(prm, lane_get<V>(va[u], k), (Op::NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f, acc0[u],
+                    acc1[u]);
+          }
+        }
+      }
+    }
+  }
+
+  double t0 = (acc0[0] + acc0[1]) + (acc0[2] + acc0[3]);
+  double t1 = (acc1[0] + acc1[1]) + (acc1[2] + acc1[3]);
+  t0 = block_sum(t0, lds);
+  if (Op::NACC >= 2) t1 = block_sum(t1, lds);
+  if (threadIdx.x == 0) {
+    if (pl.ppc == 1) {
+      op.finalize(c, t0, t1);
+    } else {
+      const size_t slot = size_t(c) * pl.ppc + (nt * pl.n_stiles + st);
+      part[slot] = t0;
+      if (Op::NACC >= 2) part[size_t(pl.C) * pl.ppc + slot] = t1;
+    }
+  }
+}
+
+template <typename Op, typename V>
+__global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl, FastDiv div_s, Op op,
+                                                                   const float *__restrict__ a,
+                                                                   const float *__restrict__ b,
+                                                                   double *__restrict__ part) {
+  constexpr int W = VecLanes<V>::n;
+  constexpr int G = 16 / W;                       // position groups owned by a thread
+  constexpr int STAGES = (Op::NIN >= 2) ? 1 : 2;  // samples loaded before any is consumed
+  __shared__ double lds[kTilePos];
+
+  const uint32_t ct = blockIdx.x % pl.n_ctiles;
+  const uint32_t nt = blockIdx.x / pl.n_ctiles;
+  const uint32_t c0 = ct * pl.CB;
+  const uint32_t cb = min(pl.CB, pl.C - c0);
+  const uint32_t LG = (cb * pl.S) / uint32_t(W);
+  const uint32_t n0 = nt * pl.NB;
+  const uint32_t n1 = min(pl.N, n0 + pl.NB);
+  const size_t CS = size_t(pl.C) * pl.S;
+  const size_t p0 = size_t(c0) * pl.S;
+
+  double acc0[G][W], acc1[G][W];
+  typename Op::Param prm[G][W];
+  bool valid[G];
+#pragma unroll
+  for (int i = 0; i < G; ++i) {
+    const uint32_t j = threadIdx.x + uint32_t(i) * kBlock;
+    valid[i] = j < LG;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      acc0[i][k] = acc1[i][k] = 0.0;
+      // positions past the tile read channel c0's parameters and are never used
+      const uint32_t pos = valid[i] ? j * uint32_t(W) + uint32_t(k) : 0u;
+      prm[i][k] = op.load(c0 + div_s.div(pos));
+    }
+  }
+
+  for (uint32_t n = n0; n < n1; n += uint32_t(STAGES)) {
+    V va[STAGES][G], vb[STAGES][G];
+#pragma unroll
+    for (int sg = 0; sg < STAGES; ++sg) {
+      if (n + uint32_t(sg) < n1) {
+        const V *pa = reinterpret_cast<const V *>(a + (size_t(n + sg) * CS + p0));
+        const V *pb = reinterpret_cast<const V *>(b + (size_t(n + sg) * CS + p0));
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+          if (valid[i]) {
+            va[sg][i] = pa[threadIdx.x + uint32_t(i) * kBlock];
+            if (Op::NIN >= 2) vb[sg][i] = pb[threadIdx.x + uint32_t(i) * kBlock];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int sg = 0; sg < STAGES; ++sg) {
+      if (n + uint32_t(sg) < n1) {
+#pragma unroll
+        for (int i = 0; i < G; ++i) {
+          if (valid[i]) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) {
+              op.term(prm[i][k], lane_get<V>(va[sg][i], k),
+                      (Op::NIN >= 2) ? lane_get<V>(vb[sg][i], k) : 0.0f, acc0[i][k], acc1[i][k]);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // fold positions to channels: tpc consecutive lanes share one channel
+  uint32_t tpc = 64;
+  while (tpc > 1 && tpc * cb > uint32_t(kBlock)) tpc >>= 1;
+  const uint32_t cl = threadIdx.x / tpc;
+  const uint32_t jj = threadIdx.x % tpc;
+  double res[2] = {0.0, 0.0};
+#pragma unroll
+  for (int q = 0; q < Op::NACC; ++q) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+      if (valid[i]) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          lds[(threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W) + uint32_t(k)] = q ? acc1[i][k] : acc0[i][k];
+        }
+      }
+    }
+    __syncthreads();
+    double s = 0.0;
+    if (cl < cb) {
+      const double *row = lds + cl * pl.S;
+      for (uint32_t ss = jj; ss < pl.S; ss += tpc) s += row[ss];
+    }
+    res[q] = group_sum(s, int(tpc));
+  }
+  if (cl < cb && jj == 0) {
+    const uint32_t c = c0 + cl;
+    if (pl.ppc == 1) {
+      op.finalize(c, res[0], res[1]);
+    } else {
+      const size_t slot = size_t(c) * pl.ppc + nt;
+      part[slot] = res[0];
+      if (Op::NACC >= 2) part[size_t(pl.C) * pl.ppc + slot] = res[1];
+    }
+  }
+}
+
+// One wave per channel adds the channel's partials: lane l takes partials
+// l, l+64, ... in order, then the lanes meet in a butterfly.
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void chan_reduce_fold_kernel(uint32_t C, uint32_t ppc, Op op,
+                                                                  const double *__restrict__ part) {
+  const uint32_t c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  if (c >= C) return;  // uniform per wave
+  double s0 = 0.0, s1 = 0.0;
+  const double *p0 = part + size_t(c) * ppc;
+  const double *p1 = p0 + size_t(C) * ppc;
+  for (uint32_t j = lane; j < ppc; j += kWave) {
+    s0 += p0[j];
+    if (Op::NACC >= 2) s1 += p1[j];
+  }
+  s0 = wave_sum(s0);
+  if (Op::NACC >= 2) s1 = wave_sum(s1);
+  if (lane == 0) op.finalize(c, s0, s1);
+}
+
+template <typename Op>
+void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
+                        const float *b, CUstream_st *stream) {
+  const uint32_t len = checked_len(S, C, N, symbol);
+  if (len == 0) return;
+  hipStream_t s = as_stream(stream);
+  const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b));
+  const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
+  if (Op::NIN < 2) b = a;
+
+  ScratchLease lease{nullptr, std::unique_lock<std::mutex>()};
+  double *part = nullptr;
+  if (pl.ppc > 1) {
+    lease = acquire_scratch(s, size_t(Op::NACC) * C * pl.ppc * sizeof(double));
+    part = static_cast<double *>(lease.ptr);
+  }
+  if (pl.whole) {
+    const FastDiv div_s(S);
+    if (pl.vec) {
+      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part);
+    } else {
+      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part);
+    }
+  } else {
+    if (pl.vec) {
+      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part);
+    } else {
+      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part);
+    }
+  }
+  note_launch(symbol);
+  if (pl.ppc > 1) {
+    const uint32_t waves_per_block = kBlock / kWave;
+    chan_reduce_fold_kernel<Op><<<(C + waves_per_block - 1) / waves_per_block, kBlock, 0, s>>>(C, pl.ppc, op, part);
+    note_launch(symbol);
+  }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace anode

@@ -1,0 +1,162 @@
+// Shared host/device helpers for the gfx950 kernels: vector types, exact
+// division by launch-invariant divisors, wave64 / workgroup reductions,
+// launch geometry and the per-stream scratch cache.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <mutex>
+
+// Layout fixed by the reference (routines_gpu/common.cuh:65-66, src/ffi.rs:28-33).
+struct KernelConfig {
+  uint32_t block_sz;
+  uint32_t max_block_ct;
+};
+struct CUstream_st;
+
+#define ANODE_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace anode {
+
+constexpr int kWave = 64;    // CDNA wavefront width
+constexpr int kBlock = 256;  // workgroup size of every kernel here: 4 waves, one per SIMD
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+static inline hipStream_t as_stream(CUstream_st *s) { return reinterpret_cast<hipStream_t>(s); }
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+// ---------------------------------------------------------------------------
+// Exact unsigned division by a divisor fixed at launch (Granlund-Montgomery,
+// round-up method): q = (t + ((n - t) >> sh1)) >> sh2 with t = mulhi(m, n).
+// Valid for every n in [0, 2^32) and every d in [1, 2^32).
+// ---------------------------------------------------------------------------
+struct FastDiv {
+  uint32_t d, m, sh1, sh2;
+
+  FastDiv() : d(1), m(1), sh1(0), sh2(0) {}
+  explicit FastDiv(uint32_t divisor) : d(divisor) {
+    uint32_t l = 0;
+    while (l < 32 && (uint64_t(1) << l) < divisor) ++l;  // l = ceil(log2 d)
+    const uint64_t two_l = uint64_t(1) << l;
+    m = uint32_t(((two_l - divisor) << 32) / divisor + 1);
+    sh1 = l < 1 ? l : 1;
+    sh2 = l < 1 ? 0 : l - 1;
+  }
+
+  __host__ __device__ inline uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t t = __umulhi(m, n);
+#else
+    const uint32_t t = uint32_t((uint64_t(m) * n) >> 32);
+#endif
+    return (t + ((n - t) >> sh1)) >> sh2;
+  }
+  __host__ __device__ inline void divmod(uint32_t n, uint32_t &q, uint32_t &r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Device-side reductions.  Every lane of the wave must take part.
+// ---------------------------------------------------------------------------
+#if defined(__HIPCC__)
+
+template <typename T>
+__device__ inline T wave_sum(T v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over aligned groups of `width` lanes (width a power of two <= 64).
+template <typename T>
+__device__ inline T group_sum(T v, int width) {
+  for (int off = width >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ inline float group_max(float v, int width) {
+  for (int off = width >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Workgroup sum for kBlock threads: wave butterflies, then the per-wave
+// results meet in LDS and are added in wave order.  `lds` holds kBlock/kWave
+// values.  The result is valid in every thread.  Ends with a barrier, so `lds`
+// may be reused at once.
+template <typename T>
+__device__ inline T block_sum(T v, T *lds) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+  __syncthreads();
+  T total = lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / kWave; ++w) total += lds[w];
+  __syncthreads();
+  return total;
+}
+
+#endif  // __HIPCC__
+
+// ---------------------------------------------------------------------------
+// Host runtime (runtime.hip)
+// ---------------------------------------------------------------------------
+
+// Compute units of the current device (cached per device).
+int device_cu_count();
+
+// Tunable launch parameters; defaults are set in runtime.hip and may be
+// changed at run time through anode_gpu_set_tuning().
+struct Tuning {
+  int flat_wg_per_cu;     // resident workgroups per CU targeted by streaming maps
+  int flat_unroll;        // independent 16-byte groups per thread and loop trip
+  int reduce_wg_target;   // workgroups a per-channel reduction aims to launch
+  int nontemporal;        // 1: streaming stores bypass the caches
+};
+Tuning &tuning();
+
+// Grid size for a grid-stride streaming kernel over `work_items` units of
+// per-thread work: enough workgroups to cover the items once, capped at
+// flat_wg_per_cu resident workgroups per CU.
+uint32_t stream_grid(uint64_t work_items, int items_per_thread);
+
+// Aborts with a message naming `symbol` unless cfg->block_sz is a power of
+// two: the contract of the reference's reduction entry points
+// (e.g. routines_gpu/batch_norm.cu:68).
+void require_pow2_block(const KernelConfig *cfg, const char *symbol);
+
+// dim0*dim1*dim2 as a 32-bit count; aborts with a message when it does not
+// fit (the reference's callers guard this: src/ops_gpu.rs:57-61).
+uint32_t checked_len(uint64_t a, uint64_t b, uint64_t c, const char *symbol);
+
+// Records the status of the launch just made (hipGetLastError) for
+// anode_gpu_take_last_error() and prints it to stderr on failure.
+void note_launch(const char *symbol);
+
+// A device buffer private to (current device, stream), grown on demand and
+// kept for the life of the process.  The lease holds the cache's lock: keep it
+// alive until every kernel that uses the buffer has been enqueued, so that two
+// host threads sharing a stream cannot interleave their launches.
+struct ScratchLease {
+  void *ptr;
+  std::unique_lock<std::mutex> lock;
+};
+ScratchLease acquire_scratch(hipStream_t stream, size_t bytes);
+
+}  // namespace anode

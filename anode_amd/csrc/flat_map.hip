@@ -1,0 +1,277 @@
+// Elementwise maps over flat packed arrays: the flat_map family, the two-input
+// join, u8 -> 32-bit widening (upcast, dequantize) and the additive f32 -> u8
+// quantiser.
+//
+// Data path: every lane moves 16 bytes per access (global_load/store_dwordx4),
+// consecutive lanes touch consecutive 16-byte groups, and each thread keeps
+// UNROLL independent groups in flight before the first store.  Arrays whose
+// pointers are not 16-byte aligned take the same kernels with one element per
+// lane.  All maps read an element before writing the same index, so an output
+// that aliases an input at equal index is safe.
+#include "common.hpp"
+
+#include <cmath>
+
+namespace anode {
+namespace {
+
+// ---- functors: out = f(a[, b]) -------------------------------------------------
+// Arithmetic follows routines_gpu/flat_map.cu and flat_join.cu literally; the file
+// is compiled with -ffp-contract=off so only the fmaf() written here is fused.
+
+struct CopyMap { __device__ float operator()(float x, float) const { return x; } };
+struct ModulusMap { __device__ float operator()(float x, float) const { return fabsf(x); } };
+struct SquareMap { __device__ float operator()(float x, float) const { return x * x; } };
+struct SqrtMap { __device__ float operator()(float x, float) const { return sqrtf(x); } };
+// ReLU by multiplication (flat_map.cu:175-178): negative x gives -0, -inf gives NaN.
+struct PositiveClipMap { __device__ float operator()(float x, float) const { return x * float(x > 0.0f); } };
+struct LogisticMap { __device__ float operator()(float x, float) const { return 1.0f / (1.0f + expf(-x)); } };
+struct UnitStepMap { __device__ float operator()(float x, float) const { return float(x > 0.0f); } };
+struct NormalCdfMap {
+  __device__ float operator()(float x, float) const { return 0.5f * (1.0f + erff(x * 0.7071067811865475f)); }
+};
+struct TanhMap { __device__ float operator()(float x, float) const { return tanhf(x); } };
+struct Rcosh2Map {
+  __device__ float operator()(float x, float) const {
+    const float ch = coshf(x);
+    return 1.0f / (ch * ch);
+  }
+};
+struct LeakyReluMap {
+  float c;
+  __device__ float operator()(float x, float) const {
+    const float mask = float(x > 0.0f);
+    return fmaf(1.0f - mask, c, mask) * x;
+  }
+};
+// backward maps: a = dy, b = y
+struct LeakyReluBwdMap {
+  float c;
+  __device__ float operator()(float dy, float y) const {
+    const float mask = float(y > 0.0f);
+    return fmaf(1.0f - mask, c, mask) * dy;
+  }
+};
+struct PositiveClipBwdMap { __device__ float operator()(float dy, float y) const { return dy * float(y > 0.0f); } };
+struct LogisticBwdMap { __device__ float operator()(float dy, float y) const { return dy * y * (1.0f - y); } };
+// flat_join.cu:31-35: a = x1, b = x2
+struct CopyUnitStepProductJoin { __device__ float operator()(float x1, float x2) const { return x1 * float(x2 > 0.0f); } };
+
+template <typename V> struct Lanes;
+template <> struct Lanes<float> { static constexpr int n = 1; };
+template <> struct Lanes<f32x4> { static constexpr int n = 4; };
+
+template <typename Op>
+__device__ inline float apply_vec(const Op &op, float a, float b) { return op(a, b); }
+template <typename Op>
+__device__ inline f32x4 apply_vec(const Op &op, f32x4 a, f32x4 b) {
+  f32x4 r;
+  r.x = op(a.x, b.x);
+  r.y = op(a.y, b.y);
+  r.z = op(a.z, b.z);
+  r.w = op(a.w, b.w);
+  return r;
+}
+
+template <typename V>
+__device__ inline void store_vec(V *p, V v, bool nontemporal) {
+  if (nontemporal) {
+    __builtin_nontemporal_store(v, p);
+  } else {
+    *p = v;
+  }
+}
+
+// n_groups groups of Lanes<V>::n elements, then `tail` single elements that
+// start at element n_groups * Lanes<V>::n (handled by workgroup 0).
+template <typename V, int NIN, int UNROLL, typename Op>
+__global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uint32_t tail, Op op,
+                                                          const float *a_, const float *b_,
+                                                          float *out_, int nontemporal) {
+  // no __restrict__: out_ may alias a_ or b_ at equal index
+  const V *a = reinterpret_cast<const V *>(a_);
+  const V *b = reinterpret_cast<const V *>(b_);
+  V *out = reinterpret_cast<V *>(out_);
+  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
+  const uint32_t stride = gridDim.x * kTile;
+  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+    V va[UNROLL], vb[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) {
+        va[u] = a[g];
+        vb[u] = (NIN == 2) ? b[g] : va[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) store_vec(&out[g], apply_vec(op, va[u], vb[u]), nontemporal != 0);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * uint32_t(Lanes<V>::n) + threadIdx.x;
+    const float x = a_[i];
+    const float y = (NIN == 2) ? b_[i] : x;
+    out_[i] = op(x, y);
+  }
+}
+
+template <int NIN, typename Op>
+void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, const float *b, float *out,
+                     CUstream_st *stream) {
+  if (len == 0) return;
+  const Tuning &t = tuning();
+  const bool vec = aligned16(a) && aligned16(out) && (NIN == 1 || aligned16(b));
+  hipStream_t s = as_stream(stream);
+  if (vec) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    if (t.flat_unroll >= 8) {
+      flat_map_kernel<f32x4, NIN, 8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+    } else if (t.flat_unroll >= 4) {
+      flat_map_kernel<f32x4, NIN, 4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+    } else {
+      flat_map_kernel<f32x4, NIN, 2, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+    }
+  } else {
+    flat_map_kernel<float, NIN, 4, Op><<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, op, a, b, out, 0);
+  }
+  note_launch(symbol);
+}
+
+// ---- u8 -> 32-bit widening -----------------------------------------------------
+
+struct UpcastOp {
+  typedef uint32_t out_t;
+  typedef u32x4 out4_t;
+  __device__ uint32_t operator()(uint32_t q) const { return q; }
+};
+// quantize.cu:30-32: scale = (hi - lo) / 255; y = float(x) * scale + lo as one fma
+struct DequantizeOp {
+  typedef float out_t;
+  typedef f32x4 out4_t;
+  float scale, lo;
+  __device__ float operator()(uint32_t q) const { return fmaf(float(q), scale, lo); }
+};
+
+// Vector form: each lane loads one dword (4 codes) and stores 16 bytes, so a
+// wave reads 256 contiguous bytes and writes 1 KiB contiguous bytes per access.
+template <int UNROLL, typename Op>
+__global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, uint32_t tail, Op op,
+                                                            const uint8_t *__restrict__ x,
+                                                            typename Op::out_t *__restrict__ y,
+                                                            int nontemporal) {
+  typedef typename Op::out4_t O4;
+  const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
+  O4 *y4 = reinterpret_cast<O4 *>(y);
+  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
+  const uint32_t stride = gridDim.x * kTile;
+  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+    uint32_t w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) w[u] = x4[g];
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      if (g < n_groups) {
+        O4 r;
+        r.x = op(w[u] & 0xffu);
+        r.y = op((w[u] >> 8) & 0xffu);
+        r.z = op((w[u] >> 16) & 0xffu);
+        r.w = op(w[u] >> 24);
+        store_vec(&y4[g], r, nontemporal != 0);
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * 4u + threadIdx.x;
+    y[i] = op(uint32_t(x[i]));
+  }
+}
+
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void widen_u8_scalar_kernel(uint32_t len, Op op,
+                                                                 const uint8_t *__restrict__ x,
+                                                                 typename Op::out_t *__restrict__ y) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = op(uint32_t(x[i]));
+}
+
+template <typename Op>
+void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, typename Op::out_t *y,
+                     CUstream_st *stream) {
+  if (len == 0) return;
+  const Tuning &t = tuning();
+  hipStream_t s = as_stream(stream);
+  if (aligned4(x) && aligned16(y)) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    if (t.flat_unroll >= 8) {
+      widen_u8x4_kernel<8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, x, y, t.nontemporal);
+    } else {
+      widen_u8x4_kernel<4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, x, y, t.nontemporal);
+    }
+  } else {
+    widen_u8_scalar_kernel<Op><<<stream_grid(len, 1), kBlock, 0, s>>>(len, op, x, y);
+  }
+  note_launch(symbol);
+}
+
+}  // namespace
+}  // namespace anode
+
+using namespace anode;
+
+#define ANODE_FLAT_MAP1(SYMBOL, OP)                                                              \
+  ANODE_EXPORT void SYMBOL(uint32_t len, const float *x, float *y, const KernelConfig *,       \
+                           CUstream_st *stream) {                                                \
+    launch_flat_map<1>(#SYMBOL, len, OP{}, x, x, y, stream);                                     \
+  }
+
+#define ANODE_FLAT_MAP2(SYMBOL, OP)                                                              \
+  ANODE_EXPORT void SYMBOL(uint32_t len, const float *a, const float *b, float *out,            \
+                           const KernelConfig *, CUstream_st *stream) {                          \
+    launch_flat_map<2>(#SYMBOL, len, OP{}, a, b, out, stream);                                   \
+  }
+
+ANODE_FLAT_MAP1(anode_gpu_copy_flat_map_f32, CopyMap)
+ANODE_FLAT_MAP1(anode_gpu_modulus_flat_map_f32, ModulusMap)
+ANODE_FLAT_MAP1(anode_gpu_square_flat_map_f32, SquareMap)
+ANODE_FLAT_MAP1(anode_gpu_sqrt_flat_map_f32, SqrtMap)
+ANODE_FLAT_MAP1(anode_gpu_positive_clip_flat_map_f32, PositiveClipMap)
+ANODE_FLAT_MAP1(anode_gpu_logistic_flat_map_f32, LogisticMap)
+ANODE_FLAT_MAP1(anode_gpu_unit_step_flat_map_f32, UnitStepMap)
+ANODE_FLAT_MAP1(anode_gpu_normal_cdf_flat_map_f32, NormalCdfMap)
+ANODE_FLAT_MAP1(anode_gpu_tanh_flat_map_f32, TanhMap)
+ANODE_FLAT_MAP1(anode_gpu_rcosh2_flat_map_f32, Rcosh2Map)
+
+ANODE_FLAT_MAP2(anode_gpu_positive_clip_flat_map_bwd_f32, PositiveClipBwdMap)
+ANODE_FLAT_MAP2(anode_gpu_logistic_flat_map_bwd_f32, LogisticBwdMap)
+ANODE_FLAT_MAP2(anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32, CopyUnitStepProductJoin)
+
+ANODE_EXPORT void anode_gpu_leaky_relu_flat_map_f32(uint32_t len, float c, const float *x, float *y,
+                                                    const KernelConfig *, CUstream_st *stream) {
+  launch_flat_map<1>("anode_gpu_leaky_relu_flat_map_f32", len, LeakyReluMap{c}, x, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_leaky_relu_flat_map_bwd_f32(uint32_t len, float c, const float *dy,
+                                                        const float *y, float *dx, const KernelConfig *,
+                                                        CUstream_st *stream) {
+  launch_flat_map<2>("anode_gpu_leaky_relu_flat_map_bwd_f32", len, LeakyReluBwdMap{c}, dy, y, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_upcast_u8_packed_u32(uint32_t len, const uint8_t *x, uint32_t *y,
+                                                 const KernelConfig *, CUstream_st *stream) {
+  launch_widen_u8("anode_gpu_upcast_u8_packed_u32", len, UpcastOp{}, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_dequantize_u8_packed_f32(uint32_t len, float lo, float hi, const uint8_t *x,
+                                                     float *y, const KernelConfig *, CUstream_st *stream) {
+  // the scale is formed on the host exactly as the kernel preamble of
+  // quantize.cu:30 forms it: an fp32 subtraction and an fp32 division
+  const float scale = (hi - lo) / 255.0f;
+  launch_widen_u8("anode_gpu_dequantize_u8_packed_f32", len, DequantizeOp{scale, lo}, x, y, stream);
+}

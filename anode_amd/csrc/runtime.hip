@@ -1,0 +1,226 @@
+// Host-side runtime shared by all entry points: device queries, launch
+// geometry, the per-(device, stream) scratch cache and error bookkeeping.
+#include "chan_reduce.hpp"
+#include "common.hpp"
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <utility>
+
+namespace anode {
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cu_count[kMaxDevices];
+std::atomic<int> g_last_error{0};
+
+struct ScratchBuf {
+  void *ptr = nullptr;
+  size_t cap = 0;
+};
+std::mutex g_scratch_mutex;
+std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch;
+
+Tuning g_tuning = {
+    /*flat_wg_per_cu=*/8,
+    /*flat_unroll=*/4,
+    /*reduce_wg_target=*/2048,
+    /*nontemporal=*/0,
+};
+
+}  // namespace
+
+int device_cu_count() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+  int n = g_cu_count[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    n = 256;  // MI355X
+  }
+  g_cu_count[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
+Tuning &tuning() { return g_tuning; }
+
+uint32_t stream_grid(uint64_t work_items, int items_per_thread) {
+  const uint64_t per_block = uint64_t(kBlock) * uint64_t(items_per_thread > 0 ? items_per_thread : 1);
+  uint64_t blocks = (work_items + per_block - 1) / per_block;
+  const uint64_t cap = uint64_t(device_cu_count()) * uint64_t(g_tuning.flat_wg_per_cu);
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return uint32_t(blocks);
+}
+
+void require_pow2_block(const KernelConfig *cfg, const char *symbol) {
+  const uint32_t b = cfg->block_sz;
+  if (b == 0 || (b & (b - 1)) != 0) {
+    std::fprintf(stderr, "%s: KernelConfig.block_sz = %u is not a power of two\n", symbol, b);
+    std::abort();
+  }
+}
+
+uint32_t checked_len(uint64_t a, uint64_t b, uint64_t c, const char *symbol) {
+  // a, b, c < 2^32, so a*b cannot overflow 64 bits; guard the second product.
+  const uint64_t ab = a * b;
+  if (ab > 0xffffffffull || ab * c > 0xffffffffull) {
+    std::fprintf(stderr, "%s: %llu x %llu x %llu elements do not fit a 32-bit index\n", symbol,
+                 (unsigned long long)a, (unsigned long long)b, (unsigned long long)c);
+    std::abort();
+  }
+  return uint32_t(ab * c);
+}
+
+void note_launch(const char *symbol) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    g_last_error.store(int(e), std::memory_order_relaxed);
+    std::fprintf(stderr, "%s: launch failed: %s\n", symbol, hipGetErrorString(e));
+  }
+}
+
+namespace {
+uint32_t ceil_div_u32(uint64_t a, uint64_t b) { return uint32_t((a + b - 1) / b); }
+uint32_t gcd_u32(uint32_t a, uint32_t b) {
+  while (b) {
+    const uint32_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a;
+}
+}  // namespace
+
+ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target) {
+  ReducePlan p{};
+  p.S = S;
+  p.C = C;
+  p.N = N;
+  if (S == 0 || C == 0 || N == 0) return p;
+  const uint64_t total = uint64_t(S) * C * N;
+  // elements a tile aims to read: enough tiles to fill the chip, but never so
+  // small that the per-tile epilogue dominates
+  uint64_t per_tile = total / (wg_target ? wg_target : 1);
+  if (per_tile < 16384) per_tile = 16384;
+
+  if (S > kTilePos) {
+    p.whole = 0;
+    p.CB = 1;
+    p.n_ctiles = C;
+    p.vec = (ptrs_aligned && S % 4 == 0) ? 1 : 0;
+    if (uint64_t(S) >= 2 * per_tile) {
+      p.n_stiles = ceil_div_u32(S, per_tile);
+      p.SB = (ceil_div_u32(S, p.n_stiles) + 3u) & ~3u;
+      p.n_stiles = ceil_div_u32(S, p.SB);
+      p.NB = 1;
+    } else {
+      p.n_stiles = 1;
+      p.SB = S;
+      uint64_t nb = per_tile / S;
+      if (nb < 1) nb = 1;
+      if (nb > N) nb = N;
+      p.NB = uint32_t(nb);
+    }
+  } else {
+    p.whole = 1;
+    p.SB = S;
+    p.n_stiles = 1;
+    uint32_t cb = kTilePos / S;
+    if (cb > kMaxTileChans) cb = kMaxTileChans;
+    if (cb > C) cb = C;
+    bool vec = ptrs_aligned && (uint64_t(C) * S) % 4 == 0;
+    if (vec && cb != C) {
+      // every tile must start on a 16-byte boundary: CB*S a multiple of 4
+      const uint32_t unit = 4 / gcd_u32(S, 4);
+      if (cb >= unit) {
+        cb -= cb % unit;
+      } else {
+        vec = false;
+      }
+    }
+    p.CB = cb;
+    p.vec = vec ? 1 : 0;
+    p.n_ctiles = ceil_div_u32(C, cb);
+    uint64_t nb = per_tile / (uint64_t(cb) * S);
+    if (nb < 1) nb = 1;
+    if (nb > N) nb = N;
+    p.NB = uint32_t(nb);
+  }
+  p.n_ntiles = ceil_div_u32(N, p.NB);
+  p.NB = ceil_div_u32(N, p.n_ntiles);  // balance the samples over the tiles
+  p.n_ntiles = ceil_div_u32(N, p.NB);
+  p.ppc = p.n_stiles * p.n_ntiles;
+  p.grid = p.n_ctiles * p.n_stiles * p.n_ntiles;
+  return p;
+}
+
+ScratchLease acquire_scratch(hipStream_t stream, size_t bytes) {
+  ScratchLease lease{nullptr, std::unique_lock<std::mutex>(g_scratch_mutex)};
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  ScratchBuf &buf = g_scratch[std::make_pair(dev, stream)];
+  if (buf.cap < bytes) {
+    // Grow geometrically.  The previous buffer may still be read by kernels in
+    // flight on this stream, so it is not freed: it stays allocated until the
+    // process ends (bounded by the doubling).
+    size_t cap = buf.cap ? buf.cap : size_t(1) << 16;
+    while (cap < bytes) cap <<= 1;
+    void *p = nullptr;
+    const hipError_t e = hipMalloc(&p, cap);
+    if (e != hipSuccess) {
+      g_last_error.store(int(e), std::memory_order_relaxed);
+      std::fprintf(stderr, "anode_routines_gpu: cannot allocate %zu bytes of reduction scratch: %s\n",
+                   cap, hipGetErrorString(e));
+      std::abort();
+    }
+    buf.ptr = p;
+    buf.cap = cap;
+  }
+  lease.ptr = buf.ptr;
+  return lease;
+}
+
+}  // namespace anode
+
+ANODE_EXPORT int anode_gpu_take_last_error(void) {
+  return anode::g_last_error.exchange(0, std::memory_order_relaxed);
+}
+
+ANODE_EXPORT uint32_t anode_gpu_reference_symbol_count(void) { return 46; }
+
+// Host-only view of the reduction tiling for a [S, C, N] array, as 12 words:
+// whole, CB, SB, n_ctiles, n_stiles, NB, n_ntiles, ppc, vec, grid, 0, 0.
+ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int ptrs_aligned,
+                                        uint32_t *out12) {
+  const anode::ReducePlan p =
+      anode::plan_chan_reduce(S, C, N, ptrs_aligned != 0, uint32_t(anode::tuning().reduce_wg_target));
+  const uint32_t v[12] = {p.whole, p.CB, p.SB, p.n_ctiles, p.n_stiles, p.NB, p.n_ntiles, p.ppc, p.vec, p.grid, 0, 0};
+  std::memcpy(out12, v, sizeof(v));
+}
+
+// Host-only check of the exact-division helper: returns n / d computed the way
+// the kernels compute it.
+ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return anode::FastDiv(d).div(n); }
+
+// Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal.
+// Returns the previous value, or -1 for an unknown knob.  A negative value
+// only reads.
+ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
+  anode::Tuning &t = anode::tuning();
+  int *slot = nullptr;
+  switch (knob) {
+    case 0: slot = &t.flat_wg_per_cu; break;
+    case 1: slot = &t.flat_unroll; break;
+    case 2: slot = &t.reduce_wg_target; break;
+    case 3: slot = &t.nontemporal; break;
+    default: return -1;
+  }
+  const int old = *slot;
+  if (value >= 0) *slot = value;
+  return old;
+}

@@ -1,0 +1,509 @@
+// Softmax with the categorical negative log-likelihood gather and its backward.
+//
+// Row form  [K classes (fastest), R rows]: the reduced axis is contiguous.
+//   K <= 64     : a row lives in a power-of-two group of lanes, several rows per wave;
+//   K <= 2048   : one wave per row, the row held in registers (lane l owns k = l, l+64, ...);
+//   larger K    : one workgroup per row, online max/sum pass then a normalising pass.
+// N-d form  [P pixels (fastest), C classes, N]: the reduced axis has stride P.
+//   One thread owns 4 consecutive pixels (16-byte accesses, coalesced across the
+//   wave), holds the C values of its pixels in registers and so reads x once.
+// Every reduction order is fixed by the geometry, so results are reproducible.
+// The block and the deterministic entry points of the reference share one
+// implementation here and accept any K.
+#include "chan_map.hpp"
+#include "common.hpp"
+
+#include <cmath>
+
+namespace anode {
+namespace {
+
+constexpr float kNegInf = -__builtin_huge_valf();
+
+// ---------------------------------------------------------------------------
+// row softmax
+// ---------------------------------------------------------------------------
+
+// K <= 64.  G = lanes per row (power of two >= K), log2g its logarithm.
+__global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K, uint32_t R, uint32_t log2g,
+                                                                     const float *__restrict__ x,
+                                                                     float *__restrict__ y) {
+  const uint32_t G = 1u << log2g;
+  const uint32_t rows_per_wave = uint32_t(kWave) >> log2g;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t sub = lane >> log2g;
+  const uint32_t k = lane & (G - 1);
+  const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint32_t n_waves = gridDim.x * (kBlock / kWave);
+  // the loop bound depends on the wave only, so all 64 lanes reach every shuffle
+  for (uint32_t r0 = wave * rows_per_wave; r0 < R; r0 += n_waves * rows_per_wave) {
+    const uint32_t r = r0 + sub;
+    const bool valid = (k < K) && (r < R);
+    const size_t idx = size_t(r) * K + k;
+    const float v = valid ? x[idx] : kNegInf;
+    const float m = group_max(v, int(G));
+    const float z = valid ? expf(v - m) : 0.0f;
+    const float s = group_sum(z, int(G));
+    if (valid) y[idx] = z / s;
+  }
+}
+
+// 64 < K <= 64 * VPL: one wave per row, VPL values per lane.
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
+                                                                  const float *__restrict__ x,
+                                                                  float *__restrict__ y) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint32_t n_waves = gridDim.x * (kBlock / kWave);
+  for (uint32_t r = wave; r < R; r += n_waves) {
+    const float *xr = x + size_t(r) * K;
+    float *yr = y + size_t(r) * K;
+    float v[VPL];
+    float m = kNegInf;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const uint32_t k = lane + uint32_t(i) * kWave;
+      v[i] = (k < K) ? xr[k] : kNegInf;
+      m = fmaxf(m, v[i]);
+    }
+    m = wave_max(m);
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const uint32_t k = lane + uint32_t(i) * kWave;
+      v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
+      s += v[i];
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const uint32_t k = lane + uint32_t(i) * kWave;
+      if (k < K) yr[k] = v[i] / s;
+    }
+  }
+}
+
+// Merge two (max, sum-of-exp) pairs.  A side that has seen nothing carries
+// (-inf, 0) and must not produce exp(-inf - -inf).
+__device__ inline void online_merge(float &m, float &s, float m2, float s2) {
+  const float mm = fmaxf(m, m2);
+  const float a = (m == mm) ? s : s * expf(m - mm);
+  const float b = (m2 == mm) ? s2 : s2 * expf(m2 - mm);
+  s = ((s == 0.0f) ? 0.0f : a) + ((s2 == 0.0f) ? 0.0f : b);
+  m = mm;
+}
+
+// any K: one workgroup per row
+__global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, uint32_t R,
+                                                                   const float *__restrict__ x,
+                                                                   float *__restrict__ y) {
+  __shared__ float lds_m[kBlock / kWave], lds_s[kBlock / kWave];
+  for (uint32_t r = blockIdx.x; r < R; r += gridDim.x) {
+    const float *xr = x + size_t(r) * K;
+    float *yr = y + size_t(r) * K;
+    float m = kNegInf, s = 0.0f;
+    for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
+      const float v = xr[k];
+      if (v > m) {
+        s = (s == 0.0f) ? 1.0f : fmaf(s, expf(m - v), 1.0f);
+        m = v;
+      } else if (!(v == kNegInf && m == kNegInf)) {
+        // a -inf seen before any larger value adds exp(-inf - max) = 0
+        s += expf(v - m);
+      }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      const float m2 = __shfl_xor(m, off, kWave);
+      const float s2 = __shfl_xor(s, off, kWave);
+      online_merge(m, s, m2, s2);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      lds_m[threadIdx.x / kWave] = m;
+      lds_s[threadIdx.x / kWave] = s;
+    }
+    __syncthreads();
+    m = lds_m[0];
+    s = lds_s[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; ++w) online_merge(m, s, lds_m[w], lds_s[w]);
+    __syncthreads();
+    for (uint32_t k = threadIdx.x; k < K; k += kBlock) yr[k] = expf(xr[k] - m) / s;
+  }
+}
+
+void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float *x, float *y,
+                         CUstream_st *stream) {
+  (void)checked_len(K, R, 1, symbol);
+  if (K == 0 || R == 0) return;
+  hipStream_t s = as_stream(stream);
+  const uint32_t max_blocks = uint32_t(device_cu_count()) * 8u;
+  constexpr uint32_t kWavesPerBlock = kBlock / kWave;
+  if (K <= 64) {
+    uint32_t log2g = 0;
+    while ((1u << log2g) < K) ++log2g;
+    const uint32_t rows_per_block = kWavesPerBlock * (64u >> log2g);
+    uint32_t blocks = (R + rows_per_block - 1) / rows_per_block;
+    if (blocks > max_blocks) blocks = max_blocks;
+    softmax_row_subwave_kernel<<<blocks, kBlock, 0, s>>>(K, R, log2g, x, y);
+  } else if (K <= 2048) {
+    uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > max_blocks) blocks = max_blocks;
+    if (K <= 128) {
+      softmax_row_wave_kernel<2><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else if (K <= 256) {
+      softmax_row_wave_kernel<4><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else if (K <= 512) {
+      softmax_row_wave_kernel<8><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else if (K <= 1024) {
+      softmax_row_wave_kernel<16><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else {
+      softmax_row_wave_kernel<32><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    }
+  } else {
+    uint32_t blocks = R < max_blocks ? R : max_blocks;
+    softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y);
+  }
+  note_launch(symbol);
+}
+
+// softmax.cu:144-161  nll[i] = label < K ? -log(p[label + K*i]) : NaN
+__global__ __launch_bounds__(kBlock) void softmax_cat_nll_kernel(uint32_t K, uint32_t R,
+                                                                 const float *__restrict__ p,
+                                                                 const uint32_t *__restrict__ cat,
+                                                                 float *__restrict__ nll) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < R; i += stride) {
+    const uint32_t k = cat[i];
+    nll[i] = (k < K) ? -logf(p[size_t(k) + size_t(K) * i]) : __builtin_nanf("");
+  }
+}
+
+// softmax.cu:177-195  dx[k,i] (=|+=) dy[i] * (p[k,i] - float(label[i]==k)); as a
+// channel-indexed map the "channel" is the row i and s is the class k.
+struct CatNllBwdMap {
+  const float *dy;
+  const uint32_t *cat;
+  struct Param { float dy; uint32_t label; };
+  __device__ Param load(uint32_t i) const { return Param{dy[i], cat[i]}; }
+  __device__ float value(const Param &p, float prob, float, uint32_t k) const {
+    return p.dy * (prob - float(p.label == k));
+  }
+  __device__ float accum(const Param &p, float prob, float, uint32_t k, float old) const {
+    return fmaf(p.dy, prob - float(p.label == k), old);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// N-d (channel-axis) softmax: one thread per group of W consecutive pixels
+// ---------------------------------------------------------------------------
+
+template <typename V> struct PixVec;
+template <> struct PixVec<float> {
+  static constexpr int W = 1;
+  typedef uint32_t U;
+  static __device__ float splat(float v) { return v; }
+};
+template <> struct PixVec<f32x4> {
+  static constexpr int W = 4;
+  typedef u32x4 U;
+  static __device__ f32x4 splat(float v) { return f32x4{v, v, v, v}; }
+};
+
+__device__ inline uint32_t lane_get_u(uint32_t v, int) { return v; }
+__device__ inline uint32_t lane_get_u(u32x4 v, int k) { return v[k]; }
+
+__device__ inline float vmax(float a, float b) { return fmaxf(a, b); }
+__device__ inline f32x4 vmax(f32x4 a, f32x4 b) {
+  return f32x4{fmaxf(a.x, b.x), fmaxf(a.y, b.y), fmaxf(a.z, b.z), fmaxf(a.w, b.w)};
+}
+__device__ inline float vexp(float a) { return expf(a); }
+__device__ inline f32x4 vexp(f32x4 a) { return f32x4{expf(a.x), expf(a.y), expf(a.z), expf(a.w)}; }
+__device__ inline float vrcp(float a) { return 1.0f / a; }
+__device__ inline f32x4 vrcp(f32x4 a) { return f32x4{1.0f / a.x, 1.0f / a.y, 1.0f / a.z, 1.0f / a.w}; }
+
+// Pixel-group geometry shared by the N-d kernels: group g covers pixels
+// [W*pg, W*pg + W) of sample n, with g = pg + groups_per_sample * n.
+struct PixelGrid {
+  uint32_t P, C, N;
+  uint32_t total_groups;
+  FastDiv div_gps;  // groups per sample
+};
+
+__device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint32_t &p, uint32_t &n) {
+  uint32_t q, r;
+  pg.div_gps.divmod(g, q, r);
+  n = q;
+  p = r * uint32_t(W);
+}
+
+// C <= CMAX: the pixel's classes stay in registers, x is read once.  The sum
+// of exponentials is formed class by class in index order; the normalisation
+// multiplies by one correctly rounded reciprocal per pixel.
+template <int CMAX, typename V>
+__global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
+                                                                float *__restrict__ y) {
+  constexpr int W = PixVec<V>::W;
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+    uint32_t p, n;
+    pixel_decode(pg, g, W, p, n);
+    const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
+    V v[CMAX];
+    V m = PixVec<V>::splat(kNegInf);
+#pragma unroll
+    for (int k = 0; k < CMAX; ++k) {
+      if (uint32_t(k) < pg.C) {
+        v[k] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * k);
+        m = vmax(m, v[k]);
+      }
+    }
+    V s = PixVec<V>::splat(0.0f);
+#pragma unroll
+    for (int k = 0; k < CMAX; ++k) {
+      if (uint32_t(k) < pg.C) {
+        v[k] = vexp(v[k] - m);
+        s += v[k];
+      }
+    }
+    const V inv = vrcp(s);
+#pragma unroll
+    for (int k = 0; k < CMAX; ++k) {
+      if (uint32_t(k) < pg.C) *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = v[k] * inv;
+    }
+  }
+}
+
+// any C: online max/sum pass over the classes, then a normalising pass
+template <typename V>
+__global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg, const float *__restrict__ x,
+                                                                   float *__restrict__ y) {
+  constexpr int W = PixVec<V>::W;
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+    uint32_t p, n;
+    pixel_decode(pg, g, W, p, n);
+    const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
+    V m = PixVec<V>::splat(kNegInf);
+    for (uint32_t k = 0; k < pg.C; ++k) m = vmax(m, *reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
+    V s = PixVec<V>::splat(0.0f);
+    for (uint32_t k = 0; k < pg.C; ++k) s += vexp(*reinterpret_cast<const V *>(x + base + size_t(pg.P) * k) - m);
+    const V inv = vrcp(s);
+    for (uint32_t k = 0; k < pg.C; ++k) {
+      const V z = vexp(*reinterpret_cast<const V *>(x + base + size_t(pg.P) * k) - m);
+      *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = z * inv;
+    }
+  }
+}
+
+// softmax.cu:278-298: per-pixel gather; one thread per pixel
+__global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg, const float *__restrict__ prob,
+                                                                    const uint32_t *__restrict__ cat,
+                                                                    float *__restrict__ nll) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+    uint32_t p, n;
+    pixel_decode(pg, g, 1, p, n);
+    const uint32_t k = cat[g];
+    nll[g] = (k < pg.C) ? -logf(prob[size_t(p) + size_t(pg.P) * (size_t(k) + size_t(pg.C) * n)])
+                        : __builtin_nanf("");
+  }
+}
+
+// softmax.cu:315-334: dx[p,k,n] (=|+=) dy[p,n] * (prob - float(label[p,n]==k)).
+// A thread reads dy and the label of its pixels once and walks the classes.
+template <typename V, bool ACC>
+__global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGrid pg,
+                                                                        const float *__restrict__ dy,
+                                                                        const float *__restrict__ prob,
+                                                                        const uint32_t *__restrict__ cat,
+                                                                        float *dx) {
+  constexpr int W = PixVec<V>::W;
+  typedef typename PixVec<V>::U U;
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+    uint32_t p, n;
+    pixel_decode(pg, g, W, p, n);
+    const size_t pix = size_t(p) + size_t(pg.P) * n;
+    const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
+    const V d = *reinterpret_cast<const V *>(dy + pix);
+    const U lab = *reinterpret_cast<const U *>(cat + pix);
+#pragma unroll 4
+    for (uint32_t k = 0; k < pg.C; ++k) {
+      const size_t off = base + size_t(pg.P) * k;
+      const V pr = *reinterpret_cast<const V *>(prob + off);
+      V old;
+      if (ACC) old = *reinterpret_cast<const V *>(dx + off);
+      V r;
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        const float t = lane_get<V>(pr, w) - float(lane_get_u(lab, w) == k);
+        lane_set<V>(r, w, ACC ? fmaf(lane_get<V>(d, w), t, lane_get<V>(old, w)) : lane_get<V>(d, w) * t);
+      }
+      *reinterpret_cast<V *>(dx + off) = r;
+    }
+  }
+}
+
+PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W) {
+  PixelGrid pg;
+  pg.P = P;
+  pg.C = C;
+  pg.N = N;
+  const uint32_t gps = P / uint32_t(W);
+  pg.total_groups = gps * N;
+  pg.div_gps = FastDiv(gps ? gps : 1);
+  return pg;
+}
+
+uint32_t pixel_blocks(uint32_t total_groups) {
+  const uint32_t cap = uint32_t(device_cu_count()) * 8u;
+  uint32_t blocks = (total_groups + kBlock - 1) / kBlock;
+  if (blocks > cap) blocks = cap;
+  return blocks ? blocks : 1;
+}
+
+template <typename V>
+void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, hipStream_t s) {
+  const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
+  const uint32_t blocks = pixel_blocks(pg.total_groups);
+  if (C <= 4) {
+    softmax_nd_reg_kernel<4, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  } else if (C <= 8) {
+    softmax_nd_reg_kernel<8, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  } else if (C <= 16) {
+    softmax_nd_reg_kernel<16, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  } else if (C <= 24) {
+    softmax_nd_reg_kernel<24, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  } else if (C <= 32) {
+    softmax_nd_reg_kernel<32, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  } else {
+    softmax_nd_stream_kernel<V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+  }
+}
+
+void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
+                       CUstream_st *stream) {
+  const uint32_t len = checked_len(P, C, N, symbol);
+  if (len == 0) return;
+  if (P == 1) {  // the class axis is contiguous: this is the row form
+    launch_softmax_rows(symbol, C, N, x, y, stream);
+    return;
+  }
+  hipStream_t s = as_stream(stream);
+  const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
+  if (C > 32 && C <= 128) {
+    // too many classes for four pixels per thread: one pixel per thread keeps
+    // the row in registers and is still coalesced across the wave
+    const PixelGrid pg = make_pixel_grid(P, C, N, 1);
+    const uint32_t blocks = pixel_blocks(pg.total_groups);
+    if (C <= 64) {
+      softmax_nd_reg_kernel<64, float><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    } else {
+      softmax_nd_reg_kernel<128, float><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    }
+  } else if (vec) {
+    launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
+  } else {
+    launch_softmax_nd_typed<float>(P, C, N, x, y, s);
+  }
+  note_launch(symbol);
+}
+
+template <bool ACC>
+void launch_softmax_cat_nll_bwd(const char *symbol, uint32_t K, uint32_t R, const float *dy, const float *prob,
+                                const uint32_t *cat, float *dx, CUstream_st *stream) {
+  launch_chan_map<1, ACC>(symbol, K, R, 1, CatNllBwdMap{dy, cat}, prob, nullptr, dx, stream);
+}
+
+template <bool ACC>
+void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *dy,
+                                   const float *prob, const uint32_t *cat, float *dx, CUstream_st *stream) {
+  const uint32_t len = checked_len(P, C, N, symbol);
+  if (len == 0) return;
+  if (P == 1) {
+    launch_softmax_cat_nll_bwd<ACC>(symbol, C, N, dy, prob, cat, dx, stream);
+    return;
+  }
+  hipStream_t s = as_stream(stream);
+  const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
+  if (vec) {
+    const PixelGrid pg = make_pixel_grid(P, C, N, 4);
+    softmax_nd_cat_nll_bwd_kernel<f32x4, ACC><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+  } else {
+    const PixelGrid pg = make_pixel_grid(P, C, N, 1);
+    softmax_nd_cat_nll_bwd_kernel<float, ACC><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+  }
+  note_launch(symbol);
+}
+
+}  // namespace
+}  // namespace anode
+
+using namespace anode;
+
+ANODE_EXPORT void anode_gpu_softmax_packed_block_f32(uint32_t dim0, uint32_t dim1, const float *x, float *y,
+                                                     const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_rows(__func__, dim0, dim1, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_packed_deterministic_f32(uint32_t dim0, uint32_t dim1, const float *x,
+                                                             float *y, const KernelConfig *,
+                                                             CUstream_st *stream) {
+  launch_softmax_rows(__func__, dim0, dim1, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_packed_f32(uint32_t dim0, uint32_t dim1, const float *softmax,
+                                                       const uint32_t *cat_data, float *nll,
+                                                       const KernelConfig *, CUstream_st *stream) {
+  (void)checked_len(dim0, dim1, 1, __func__);
+  if (dim1 == 0) return;
+  softmax_cat_nll_kernel<<<stream_grid(dim1, 1), kBlock, 0, as_stream(stream)>>>(dim0, dim1, softmax, cat_data, nll);
+  note_launch(__func__);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy,
+                                                           const float *softmax, const uint32_t *cat_data,
+                                                           float *dx, const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_cat_nll_bwd<false>(__func__, dim0, dim1, dy, softmax, cat_data, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32(uint32_t dim0, uint32_t dim1,
+                                                                      const float *dy, const float *softmax,
+                                                                      const uint32_t *cat_data, float *dx,
+                                                                      const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_cat_nll_bwd<true>(__func__, dim0, dim1, dy, softmax, cat_data, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
+                                                  const float *x, float *y, const KernelConfig *,
+                                                  CUstream_st *stream) {
+  launch_softmax_nd(__func__, prefix_dim, dim0, dim1, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
+                                                          const float *softmax, const uint32_t *cat_data,
+                                                          float *nll, const KernelConfig *, CUstream_st *stream) {
+  (void)checked_len(prefix_dim, dim0, dim1, __func__);
+  if (prefix_dim == 0 || dim1 == 0) return;
+  const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 1);
+  softmax_nd_cat_nll_kernel<<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
+  note_launch(__func__);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
+                                                              const float *dy, const float *softmax,
+                                                              const uint32_t *cat_data, float *dx,
+                                                              const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_nd_cat_nll_bwd<false>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_t prefix_dim, uint32_t dim0,
+                                                                         uint32_t dim1, const float *dy,
+                                                                         const float *softmax,
+                                                                         const uint32_t *cat_data, float *dx,
+                                                                         const KernelConfig *,
+                                                                         CUstream_st *stream) {
+  launch_softmax_nd_cat_nll_bwd<true>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream);
+}

@@ -1,0 +1,192 @@
+/*
+ * C ABI of the MI355X (gfx950, HIP) implementation of anode's GPU operator
+ * library.
+ *
+ * Part 1 declares the 46 entry points of the reference's
+ * routines_gpu/lib.h:32-510 with identical names, parameter order and types,
+ * so that anode's Rust bindings (build.rs:61-121 -> src/ffi.rs:35) link
+ * against this library unchanged.  Part 2 declares ADDITIVE entry points that
+ * have no counterpart in the reference (bindgen ignores them:
+ * whitelist_recursively(false), build.rs:63).
+ *
+ * Conventions shared by every entry point (reference: lib.h:27-39,
+ * common.cuh:51-67, src/ops_gpu.rs:670-679):
+ *   - all data pointers are DEVICE pointers to packed arrays; `cfg` is a HOST
+ *     pointer, read during the call;
+ *   - `stream` is the runtime's stream handle (a hipStream_t passed through the
+ *     opaque struct CUstream_st*; NULL = the null stream);
+ *   - the call enqueues work on `stream` and returns; nothing is reported;
+ *   - index order is first-index-fastest: element (i0,i1,i2) of a
+ *     [dim0,dim1,dim2] array lives at i0 + dim0*(i1 + dim1*i2)
+ *     (common.cuh:87-106).  With anode's callers (dim0,dim1,dim2) =
+ *     (W*H[*D], C, N), i.e. the memory of a contiguous NCHW / NCDHW tensor;
+ *   - dim0*dim1*dim2 must be < 2^32 (src/ops_gpu.rs:57-61);
+ *   - `*_accumulate_*` entry points add into the output instead of assigning
+ *     (common.cuh:171-193);
+ *   - entry points that the reference implements as block reductions abort
+ *     the process when cfg->block_sz is not a power of two, as the
+ *     reference's host-side assert does (e.g. batch_norm.cu:68).  Otherwise
+ *     `cfg` is a hint: launch geometry is chosen by the library.
+ */
+#ifndef ANODE_ROUTINES_GPU_H_
+#define ANODE_ROUTINES_GPU_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Layout fixed by common.cuh:65-66 and the Rust twin in src/ffi.rs:28-33:
+ *   struct KernelConfig { uint32_t block_sz; uint32_t max_block_ct; };
+ * It is left incomplete here exactly as in lib.h:27; C/C++ callers that need
+ * to build one define ANODE_DEFINE_KERNEL_CONFIG before including this file. */
+struct KernelConfig;
+struct CUstream_st;
+
+#ifdef ANODE_DEFINE_KERNEL_CONFIG
+struct KernelConfig {
+  uint32_t block_sz;
+  uint32_t max_block_ct;
+};
+#endif
+
+#define ANODE_LAUNCH_TAIL const struct KernelConfig *cfg, struct CUstream_st *stream
+
+/* ===================================================================== */
+/* Part 1: the reference ABI                                             */
+/* ===================================================================== */
+
+/* ---- batch-norm pieces (batch_norm.cu); n = float(dim0)*float(dim2) ---- */
+
+/* lib.h:32-39, batch_norm.cu:24-71.  mean[c] = (sum_{i0,i2} x) / n */
+void anode_gpu_batch_mean_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, float *mean, ANODE_LAUNCH_TAIL);
+/* lib.h:40-47, batch_norm.cu:73-109.  dx = dmean[c] / n */
+void anode_gpu_batch_mean_bwd_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dmean, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:48-55, batch_norm.cu:111-123.  dx += dmean[c] / n */
+void anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dmean, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:56-65, batch_norm.cu:125-179.  var[c] = sum (x-mean[c])^2 / n + epsilon (biased; epsilon inside) */
+void anode_gpu_batch_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, const float *mean, float *var, ANODE_LAUNCH_TAIL);
+/* lib.h:66-75, batch_norm.cu:181-222.  dx = dvar[c] * (x-mean[c]) * 2 / n */
+void anode_gpu_batch_var_bwd_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dvar, const float *x, const float *mean, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:76-85, batch_norm.cu:224-238.  dx += ... */
+void anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dvar, const float *x, const float *mean, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:86-95, batch_norm.cu:240-296.  dmean[c] = (sum (x-mean[c]) * (-2*dvar[c])) / n */
+void anode_gpu_batch_var_bwd_mean_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dvar, const float *x, const float *mean, float *dmean, ANODE_LAUNCH_TAIL);
+/* lib.h:96-105, batch_norm.cu:298-312.  dmean[c] += ... */
+void anode_gpu_batch_var_bwd_mean_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dvar, const float *x, const float *mean, float *dmean, ANODE_LAUNCH_TAIL);
+/* lib.h:106-115, batch_norm.cu:314-352.  y = (x-mean[c]) * rsqrt(var[c])   (var already holds +epsilon) */
+void anode_gpu_batch_norm_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, const float *mean, const float *var, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:116-124, batch_norm.cu:354-391.  dx = dy * rsqrt(var[c]) */
+void anode_gpu_batch_norm_bwd_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *var, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:125-133, batch_norm.cu:393-406.  dx += ... */
+void anode_gpu_batch_norm_bwd_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *var, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:134-142, batch_norm.cu:408-459.  dmean[c] = sum dy * (-rsqrt(var[c])) */
+void anode_gpu_batch_norm_bwd_mean_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *var, float *dmean, ANODE_LAUNCH_TAIL);
+/* lib.h:143-151, batch_norm.cu:461-474.  dmean[c] += ... */
+void anode_gpu_batch_norm_bwd_mean_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *var, float *dmean, ANODE_LAUNCH_TAIL);
+/* lib.h:152-162, batch_norm.cu:476-532.  dvar[c] = sum dy * (x-mean[c]) * (-0.5 * rsqrt(v) / v), v = var[c] */
+void anode_gpu_batch_norm_bwd_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, float *dvar, ANODE_LAUNCH_TAIL);
+/* lib.h:163-173, batch_norm.cu:534-549.  dvar[c] += ... */
+void anode_gpu_batch_norm_bwd_var_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, float *dvar, ANODE_LAUNCH_TAIL);
+/* lib.h:174-183, batch_norm.cu:551-603.  dvar[c] = sum -dy * y * 0.5 / var[c]   (from the normalised output y) */
+void anode_gpu_batch_norm_bwd_var_v2_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *y, const float *var, float *dvar, ANODE_LAUNCH_TAIL);
+/* lib.h:184-193, batch_norm.cu:605-619.  dvar[c] += ... */
+void anode_gpu_batch_norm_bwd_var_v2_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *y, const float *var, float *dvar, ANODE_LAUNCH_TAIL);
+
+/* ---- casts, quantisation, discrete ---- */
+
+/* lib.h:253-258, cast.cu:23-42.  y[i] = (uint32_t) x[i] */
+void anode_gpu_upcast_u8_packed_u32(uint32_t len, const uint8_t *x, uint32_t *y, ANODE_LAUNCH_TAIL);
+/* lib.h:262-269, discrete.cu:21-60.  y[i0,k,i2] = (x[i0 + dim0*i2] == k) ? 1 : 0 */
+void anode_gpu_discrete_one_hot_3d1_packed_f32(uint32_t dim0, uint32_t cat_dim1, uint32_t dim2, const uint32_t *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:397-404, quantize.cu:23-47.  y = fma(float(x), (hi-lo)/255, lo) */
+void anode_gpu_dequantize_u8_packed_f32(uint32_t len, float lo, float hi, const uint8_t *x, float *y, ANODE_LAUNCH_TAIL);
+
+/* ---- smooth F1 loss (f1.cu) ---- */
+
+/* lib.h:273-282, f1.cu:23-87.  y[k,n] = -(2*sum_i0 x*t + eps) / (sum_i0 (x+t) + eps) */
+void anode_gpu_smooth_negative_f1_loss_3d1_packed_f32(uint32_t dim0, uint32_t cat_dim1, uint32_t dim2, float epsilon, const float *x, const float *target, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:283-293, f1.cu:89-132.  dx = dy[k,n] * -(2 t (t+eps) - eps) / (x+t+eps)^2 */
+void anode_gpu_smooth_negative_f1_loss_3d1_bwd_packed_f32(uint32_t dim0, uint32_t cat_dim1, uint32_t dim2, float epsilon, const float *dy, const float *x, const float *target, float *dx, ANODE_LAUNCH_TAIL);
+
+/* ---- flat_join.cu ---- */
+
+/* lib.h:296-302, flat_join.cu:28-60.  y = x1 * float(x2 > 0) */
+void anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32(uint32_t len, const float *x1, const float *x2, float *y, ANODE_LAUNCH_TAIL);
+
+/* ---- flat_map.cu: y[i] = f(x[i]); backward maps dx[i] = g(dy[i], y[i]).
+ *      Output may alias the same-index input (in-place ReLU,
+ *      src/ops_gpu.rs:7906-7940). ---- */
+
+/* lib.h:305-311, flat_map.cu:44-52,96-106.  m = float(x>0); y = (m + (1-m)*c) * x */
+void anode_gpu_leaky_relu_flat_map_f32(uint32_t len, float c, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:312-319, flat_map.cu:60-69,108-119.  m = float(y>0); dx = (m + (1-m)*c) * dy */
+void anode_gpu_leaky_relu_flat_map_bwd_f32(uint32_t len, float c, const float *dy, const float *y, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:320-325, flat_map.cu:121-127,348-357.  y = x */
+void anode_gpu_copy_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:326-331, flat_map.cu:135-141,359-368.  y = |x| */
+void anode_gpu_modulus_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:332-337, flat_map.cu:143-150,370-379.  y = x*x */
+void anode_gpu_square_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:338-343, flat_map.cu:158-164,381-390.  y = sqrt(x), correctly rounded */
+void anode_gpu_sqrt_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:344-349, flat_map.cu:172-179,392-401.  y = x * float(x>0)   (ReLU by multiply: x<0 -> -0, -inf -> NaN) */
+void anode_gpu_positive_clip_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:350-356, flat_map.cu:187-194,403-413.  dx = dy * float(y>0) */
+void anode_gpu_positive_clip_flat_map_bwd_f32(uint32_t len, const float *dy, const float *y, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:357-362, flat_map.cu:202-209,415-424.  y = 1 / (1 + exp(-x)) */
+void anode_gpu_logistic_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:363-369, flat_map.cu:217-225,426-436.  dx = dy * y * (1-y) */
+void anode_gpu_logistic_flat_map_bwd_f32(uint32_t len, const float *dy, const float *y, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:370-375, flat_map.cu:233-240,438-447.  y = float(x>0) */
+void anode_gpu_unit_step_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:376-381, flat_map.cu:286-293,449-458.  y = 0.5 * (1 + erf(x / sqrt 2)) */
+void anode_gpu_normal_cdf_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:382-387, flat_map.cu:301-307,460-469.  y = tanh(x) */
+void anode_gpu_tanh_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:388-393, flat_map.cu:315-323,471-480.  y = 1 / cosh(x)^2 */
+void anode_gpu_rcosh2_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+
+/* ---- softmax and categorical NLL (softmax.cu).  Row form: element (k,i) of
+ *      a [dim0 classes, dim1 rows] array at k + dim0*i.  N-d form: element
+ *      (p,k,n) of [prefix_dim, dim0 classes, dim1] at p + prefix_dim*(k + dim0*n),
+ *      labels / dy / nll at p + prefix_dim*n. ---- */
+
+/* lib.h:434-440, softmax.cu:24-78.  Row softmax; the reference requires dim0 <= cfg->block_sz
+ * (caller dispatch at src/ops_gpu.rs:6153); this implementation accepts any dim0. */
+void anode_gpu_softmax_packed_block_f32(uint32_t dim0, uint32_t dim1, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:441-447, softmax.cu:80-142.  Row softmax, any dim0. */
+void anode_gpu_softmax_packed_deterministic_f32(uint32_t dim0, uint32_t dim1, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:448-455, softmax.cu:144-175.  nll[i] = label<dim0 ? -log(softmax[label + dim0*i]) : NaN */
+void anode_gpu_softmax_cat_nll_packed_f32(uint32_t dim0, uint32_t dim1, const float *softmax, const uint32_t *cat_data, float *nll, ANODE_LAUNCH_TAIL);
+/* lib.h:456-464, softmax.cu:177-210.  dx[k,i] = dy[i] * (softmax[k,i] - float(label[i]==k))   (bad label: unmasked) */
+void anode_gpu_softmax_cat_nll_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:465-473, softmax.cu:212-225.  dx += ... */
+void anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:474-481, softmax.cu:227-276.  Channel-axis softmax per pixel. */
+void anode_gpu_softmax_nd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:482-490, softmax.cu:278-313.  Per-pixel gather, NaN when label >= dim0. */
+void anode_gpu_softmax_nd_cat_nll_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *softmax, const uint32_t *cat_data, float *nll, ANODE_LAUNCH_TAIL);
+/* lib.h:491-500, softmax.cu:315-350.  dx[p,k,n] = dy[p,n] * (softmax - float(label[p,n]==k)) */
+void anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+/* lib.h:501-510, softmax.cu:352-366.  dx += ... */
+void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+
+/* ===================================================================== */
+/* Part 2: additive entry points (no counterpart in the reference)       */
+/* ===================================================================== */
+
+/* Library introspection.  No reference counterpart. */
+/* 0 when no launch made by this library has failed since the last call; otherwise the hipError_t
+ * of the most recent failed launch.  Reading clears it. */
+int anode_gpu_take_last_error(void);
+/* Number of entry points of Part 1 (46). */
+uint32_t anode_gpu_reference_symbol_count(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* ANODE_ROUTINES_GPU_H_ */
