@@ -1,0 +1,206 @@
+"""The drop-in boundary, checked without a GPU: the shared and the static
+library export, with C linkage, every entry point that include/anode_routines_gpu.h
+declares; the header declares the 46 names of the reference's routines_gpu/lib.h
+with the reference's parameter lists; host-side contracts (KernelConfig layout,
+the power-of-two assertion, exact division, tiling plans) hold.
+"""
+import ctypes
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from anode_amd import _lib
+
+# name -> parameter kinds before (cfg, stream), transcribed from routines_gpu/lib.h:32-510
+# u = uint32_t, f = float, p = device pointer
+REFERENCE_ABI = {
+    "anode_gpu_batch_mean_3d1_packed_f32": "uuupp",
+    "anode_gpu_batch_mean_bwd_3d1_packed_f32": "uuupp",
+    "anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32": "uuupp",
+    "anode_gpu_batch_var_3d1_packed_f32": "uuufppp",
+    "anode_gpu_batch_var_bwd_3d1_packed_f32": "uuupppp",
+    "anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32": "uuupppp",
+    "anode_gpu_batch_var_bwd_mean_3d1_packed_f32": "uuupppp",
+    "anode_gpu_batch_var_bwd_mean_3d1_packed_accumulate_f32": "uuupppp",
+    "anode_gpu_batch_norm_3d1_packed_f32": "uuupppp",
+    "anode_gpu_batch_norm_bwd_3d1_packed_f32": "uuuppp",
+    "anode_gpu_batch_norm_bwd_3d1_packed_accumulate_f32": "uuuppp",
+    "anode_gpu_batch_norm_bwd_mean_3d1_packed_f32": "uuuppp",
+    "anode_gpu_batch_norm_bwd_mean_3d1_packed_accumulate_f32": "uuuppp",
+    "anode_gpu_batch_norm_bwd_var_3d1_packed_f32": "uuuppppp",
+    "anode_gpu_batch_norm_bwd_var_3d1_packed_accumulate_f32": "uuuppppp",
+    "anode_gpu_batch_norm_bwd_var_v2_3d1_packed_f32": "uuupppp",
+    "anode_gpu_batch_norm_bwd_var_v2_3d1_packed_accumulate_f32": "uuupppp",
+    "anode_gpu_upcast_u8_packed_u32": "upp",
+    "anode_gpu_discrete_one_hot_3d1_packed_f32": "uuupp",
+    "anode_gpu_smooth_negative_f1_loss_3d1_packed_f32": "uuufppp",
+    "anode_gpu_smooth_negative_f1_loss_3d1_bwd_packed_f32": "uuufpppp",
+    "anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32": "uppp",
+    "anode_gpu_leaky_relu_flat_map_f32": "ufpp",
+    "anode_gpu_leaky_relu_flat_map_bwd_f32": "ufppp",
+    "anode_gpu_copy_flat_map_f32": "upp",
+    "anode_gpu_modulus_flat_map_f32": "upp",
+    "anode_gpu_square_flat_map_f32": "upp",
+    "anode_gpu_sqrt_flat_map_f32": "upp",
+    "anode_gpu_positive_clip_flat_map_f32": "upp",
+    "anode_gpu_positive_clip_flat_map_bwd_f32": "uppp",
+    "anode_gpu_logistic_flat_map_f32": "upp",
+    "anode_gpu_logistic_flat_map_bwd_f32": "uppp",
+    "anode_gpu_unit_step_flat_map_f32": "upp",
+    "anode_gpu_normal_cdf_flat_map_f32": "upp",
+    "anode_gpu_tanh_flat_map_f32": "upp",
+    "anode_gpu_rcosh2_flat_map_f32": "upp",
+    "anode_gpu_dequantize_u8_packed_f32": "uffpp",
+    "anode_gpu_softmax_packed_block_f32": "uupp",
+    "anode_gpu_softmax_packed_deterministic_f32": "uupp",
+    "anode_gpu_softmax_cat_nll_packed_f32": "uuppp",
+    "anode_gpu_softmax_cat_nll_bwd_packed_f32": "uupppp",
+    "anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32": "uupppp",
+    "anode_gpu_softmax_nd_packed_f32": "uuupp",
+    "anode_gpu_softmax_nd_cat_nll_packed_f32": "uuuppp",
+    "anode_gpu_softmax_nd_cat_nll_bwd_packed_f32": "uuupppp",
+    "anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32": "uuupppp",
+}
+
+_KIND = {ctypes.c_uint32: "u", ctypes.c_float: "f", ctypes.c_void_p: "p", ctypes.c_int: "i"}
+
+
+def _nm_defined(path, dynamic):
+    out = subprocess.run(["nm", "-D" if dynamic else "-g", "--defined-only", path], check=True,
+                         capture_output=True, text=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if " T " in line}
+
+
+def test_reference_abi_has_46_entry_points():
+    assert len(REFERENCE_ABI) == 46
+
+
+def test_header_declares_the_reference_abi_with_its_parameter_lists():
+    protos = _lib.parse_header()
+    for name, kinds in REFERENCE_ABI.items():
+        assert name in protos, f"{name} missing from the header"
+        restype, argtypes, names = protos[name]
+        assert restype is None, f"{name} must return void"
+        got = "".join(_KIND[t] for t in argtypes)
+        assert got == kinds + "pp", f"{name}: {got} != {kinds}+cfg+stream"
+        assert names[-2:] == ["cfg", "stream"]
+
+
+def test_shared_library_exports_every_declared_symbol_unmangled():
+    assert os.path.exists(_lib.LIBRARY_PATH), "run __graft_entry__.build() first"
+    exported = _nm_defined(_lib.LIBRARY_PATH, dynamic=True)
+    for name in _lib.parse_header():
+        assert name in exported, f"{name} declared but not exported"
+    assert not any(s.startswith("_Z") and "anode_gpu" in s for s in exported)
+
+
+def test_static_archive_defines_every_reference_symbol():
+    # the artefact anode's build script links by name: static lib `anode_routines_gpu` (build.rs:23)
+    assert os.path.basename(_lib.STATIC_LIBRARY_PATH) == "libanode_routines_gpu.a"
+    assert os.path.exists(_lib.STATIC_LIBRARY_PATH)
+    defined = _nm_defined(_lib.STATIC_LIBRARY_PATH, dynamic=False)
+    for name in REFERENCE_ABI:
+        assert name in defined
+
+
+def test_library_loads_and_reports_symbol_count():
+    lib = _lib.load()
+    assert lib.symbol("anode_gpu_reference_symbol_count")() == 46
+    assert ctypes.sizeof(_lib.KernelConfig) == 8
+    assert _lib.KernelConfig.block_sz.offset == 0 and _lib.KernelConfig.max_block_ct.offset == 4
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        _lib.Library(str(tmp_path / "libanode_routines_gpu.so"))
+
+
+_ABORT_SNIPPET = r"""
+import ctypes, sys
+sys.path.insert(0, {root!r})
+from anode_amd import _lib
+lib = _lib.load()
+cfg = _lib.KernelConfig({block}, 64)
+# null device pointers: the contract check comes before anything touches the GPU
+lib.symbol({name!r})(*{args!r}, ctypes.byref(cfg), None)
+print("returned")
+"""
+
+
+@pytest.mark.parametrize("name", [
+    "anode_gpu_batch_mean_3d1_packed_f32",
+    "anode_gpu_batch_var_3d1_packed_f32",
+    "anode_gpu_batch_norm_bwd_var_3d1_packed_accumulate_f32",
+    "anode_gpu_smooth_negative_f1_loss_3d1_packed_f32",
+])
+def test_reduction_entry_points_abort_on_non_power_of_two_block(name):
+    # routines_gpu/batch_norm.cu:68, f1.cu:84: assert(check_power_of_2(block_sz)) on the host
+    kinds = REFERENCE_ABI[name]
+    args = [{"u": 5, "f": 1e-5, "p": None}[k] for k in kinds]
+    code = _ABORT_SNIPPET.format(root=_lib.REPO_ROOT, block=100, name=name, args=args)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == -6, (r.returncode, r.stdout, r.stderr)
+    assert "not a power of two" in r.stderr and name in r.stderr
+    assert "returned" not in r.stdout
+
+
+def test_exact_division_helper_matches_integer_division():
+    probe = _lib.load().cdll.anode_gpu_fastdiv_probe
+    g = np.random.default_rng(0)
+    divisors = [1, 2, 3, 4, 5, 7, 19, 49, 64, 255, 256, 784, 1000, 12544, 65535, 65536, 65537, 2097152,
+                2 ** 31 - 1, 2 ** 31, 2 ** 31 + 1, 2 ** 32 - 1] + [int(v) for v in g.integers(1, 2 ** 32, 40)]
+    for d in divisors:
+        edge = [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 2 ** 32 - 1, 2 ** 32 - d, 2 ** 31, 2 ** 31 - 1]
+        ns = [n for n in edge if 0 <= n < 2 ** 32] + [int(v) for v in g.integers(0, 2 ** 32, 200)]
+        for n in ns:
+            assert probe(n, d) == n // d, (n, d)
+
+
+def _plan(S, C, N, aligned=True):
+    out = (ctypes.c_uint32 * 12)()
+    _lib.load().cdll.anode_gpu_plan_reduce(S, C, N, int(aligned), out)
+    keys = ["whole", "CB", "SB", "n_ctiles", "n_stiles", "NB", "n_ntiles", "ppc", "vec", "grid"]
+    return dict(zip(keys, list(out)[:10]))
+
+
+@pytest.mark.parametrize("S,C,N", [
+    (784, 16, 32), (12544, 64, 256), (49, 2048, 256), (2097152, 32, 2), (1, 1000, 64), (1, 1, 1), (3, 5, 7),
+    (4097, 3, 9), (4096, 1, 1), (50, 3, 2), (12321, 8, 4), (7, 300000, 2), (100000, 4, 1),
+])
+def test_reduction_tiling_covers_the_array_exactly_once(S, C, N):
+    for aligned in (True, False):
+        p = _plan(S, C, N, aligned)
+        assert p["grid"] == p["n_ctiles"] * p["n_stiles"] * p["n_ntiles"] >= 1
+        assert p["ppc"] == p["n_stiles"] * p["n_ntiles"]
+        assert (p["n_ntiles"] - 1) * p["NB"] < N <= p["n_ntiles"] * p["NB"]
+        if p["whole"]:
+            assert S <= 4096 and p["CB"] * S <= 4096 and 1 <= p["CB"] <= 256
+            assert (p["n_ctiles"] - 1) * p["CB"] < C <= p["n_ctiles"] * p["CB"]
+            assert p["n_stiles"] == 1
+            if p["vec"]:
+                assert aligned and (C * S) % 4 == 0
+                assert p["CB"] == C or (p["CB"] * S) % 4 == 0  # every tile starts on a 16-byte boundary
+        else:
+            assert S > 4096 and p["n_ctiles"] == C
+            assert (p["n_stiles"] - 1) * p["SB"] < S <= p["n_stiles"] * p["SB"]
+            if p["vec"]:
+                assert aligned and S % 4 == 0 and (p["SB"] % 4 == 0 or p["n_stiles"] == 1)
+        if not aligned:
+            assert not p["vec"]
+
+
+def test_product_package_never_reaches_the_oracle():
+    # the oracle is test infrastructure: nothing under anode_amd/ may import, load or link it
+    root = os.path.join(_lib.REPO_ROOT, "anode_amd")
+    for dirpath, _, files in os.walk(root):
+        if os.path.basename(dirpath) == "build":
+            continue
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f), "r", errors="ignore").read()
+                assert "oracle" not in text.lower(), f"{os.path.join(dirpath, f)} mentions the oracle"
+    needed = subprocess.run(["readelf", "-d", _lib.LIBRARY_PATH], capture_output=True, text=True).stdout
+    assert "oracle" not in needed

@@ -1,0 +1,164 @@
+"""GPU parity: softmax, the categorical NLL gather and its backward, row and
+n-d forms, through the C ABI against the oracle."""
+import math
+
+import numpy as np
+import pytest
+
+from gpu_util import F32, assert_bit_exact, assert_close, call, cfg, dev, empty, host
+
+pytestmark = pytest.mark.gpu
+
+ROW_ENTRY_POINTS = ["anode_gpu_softmax_packed_block_f32", "anode_gpu_softmax_packed_deterministic_f32"]
+
+
+# ---- the reference's own known-answer tests (tests/test_gpu.rs:595-736) ----
+
+@pytest.mark.parametrize("name", ROW_ENTRY_POINTS)
+def test_ref_softmax_zeros_is_exactly_one_over_32(name):
+    for rows in (1, 2):
+        y = empty(32 * rows)
+        call(name, 32, rows, dev(np.zeros(32 * rows, F32)), y)
+        assert np.all(host(y) == F32(1.0) / F32(32.0))
+
+
+def test_ref_softmax_cat_nll_known_answers(oracle):
+    p = empty(64)
+    call("anode_gpu_softmax_packed_block_f32", 32, 2, dev(np.zeros(64, F32)), p)
+    nll = empty(2)
+    call("anode_gpu_softmax_cat_nll_packed_f32", 32, 2, p, dev(np.array([12, 17], np.uint32)), nll)
+    assert_close(host(nll), [math.log(32.0)] * 2, "nll", rel=1e-6)
+    # out-of-range label: NaN, and a NaN batch sum (tests/test_gpu.rs:651-690)
+    call("anode_gpu_softmax_cat_nll_packed_f32", 32, 2, p, dev(np.array([12, 42], np.uint32)), nll)
+    h = host(nll)
+    assert np.isfinite(h[0]) and np.isnan(h[1]) and np.isnan(h.sum())
+    # adjoint of the batch sum (tests/test_gpu.rs:692-736): dx = 1/32 - [k == label], exactly
+    dx = empty(64)
+    call("anode_gpu_softmax_cat_nll_bwd_packed_f32", 32, 2, dev(np.ones(2, F32)), p,
+         dev(np.array([12, 17], np.uint32)), dx)
+    want = np.full((2, 32), F32(1.0) / F32(32.0), F32)
+    want[0, 12] -= 1
+    want[1, 17] -= 1
+    assert_bit_exact(host(dx), want.ravel(), "softmax_cat_nll_bwd closed form")
+
+
+# ---- row form ----
+
+ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), (64, 300), (65, 3), (100, 17),
+              (128, 5), (129, 4), (1000, 256), (1024, 3), (1025, 2), (2048, 2), (2049, 3), (5000, 2), (40000, 1)]
+
+
+@pytest.mark.parametrize("K,R", ROW_SHAPES)
+@pytest.mark.parametrize("name", ROW_ENTRY_POINTS)
+def test_softmax_rows(oracle, name, K, R):
+    print(f"case {name} K={K} R={R}", flush=True)
+    g = np.random.default_rng(K * 7 + R)
+    x = (2 * g.standard_normal(K * R)).astype(F32)
+    for offset in (0, 3):
+        y = empty(K * R, offset=offset)
+        # both entry points must be right for any K, whatever cfg says (dispatch at src/ops_gpu.rs:6153)
+        call(name, K, R, dev(x, offset), y, cfg=cfg(32, 16))
+        p = host(y)
+        assert_close(p, oracle.softmax(K, R, x, f64=True), f"softmax K={K}", abs_floor=1e-30)
+        assert_close(p.reshape(R, K).astype(np.float64).sum(1), np.ones(R), "rows sum to one", rel=1e-5)
+
+
+def test_softmax_rows_special_values(oracle):
+    K, R = 8, 4
+    x = np.zeros((R, K), F32)
+    x[0, :] = -np.inf
+    x[0, 3] = 1.0          # -inf entries get probability 0
+    x[1, :] = [1e30, -1e30, 0, 5, 5, 5, 5, 5]
+    x[2, 2] = np.nan       # a NaN poisons its row only (max ignores NaN, the sum does not)
+    x[3, :] = 88.0         # no overflow: the max is subtracted first
+    y = empty(K * R)
+    call("anode_gpu_softmax_packed_block_f32", K, R, dev(x), y)
+    p = host(y).reshape(R, K)
+    want = oracle.softmax(K, R, x.ravel(), f64=True).reshape(R, K)
+    assert_close(p, want, "special values", abs_floor=1e-30)
+    assert p[0, 3] == 1.0 and np.all(p[0, [0, 1, 2, 4]] == 0)
+    assert np.all(np.isnan(p[2])) and not np.any(np.isnan(p[[0, 1, 3]]))
+    # the same rows through the one-workgroup-per-row kernel (K above the register limit)
+    K2 = 3000
+    x2 = np.full((3, K2), -np.inf, F32)
+    x2[0, 7] = 2.0
+    x2[1, :] = 0.5
+    x2[1, 0] = -np.inf     # a leading -inf must not turn into NaN
+    x2[2, :] = np.linspace(-50, 50, K2)
+    y2 = empty(3 * K2)
+    call("anode_gpu_softmax_packed_deterministic_f32", K2, 3, dev(x2), y2)
+    assert_close(host(y2), oracle.softmax(K2, 3, x2.ravel(), f64=True), "block kernel special values", abs_floor=1e-30)
+
+
+@pytest.mark.parametrize("K,R", [(10, 32), (1000, 256), (7, 5), (1, 9), (300, 11)])
+def test_softmax_cat_nll_and_bwd_rows(oracle, K, R):
+    g = np.random.default_rng(K + R)
+    x = (2 * g.standard_normal(K * R)).astype(F32)
+    lab = g.integers(0, K, R).astype(np.uint32)
+    if R > 4:
+        lab[2] = K          # first out-of-range value
+        lab[4] = 0xFFFFFFFF
+    dy = g.standard_normal(R).astype(F32)
+    old = g.standard_normal(K * R).astype(F32)
+    for offset in (0, 1):
+        p_d = empty(K * R, offset=offset)
+        call("anode_gpu_softmax_packed_deterministic_f32", K, R, dev(x, offset), p_d)
+        p = host(p_d)
+        nll = empty(R, offset=offset)
+        call("anode_gpu_softmax_cat_nll_packed_f32", K, R, p_d, dev(lab, offset), nll)
+        # label gather: the index is exact, so nll must equal -log of exactly that stored probability
+        idx = oracle.softmax_cat_gather_index(K, R, lab)
+        ok = idx != np.iinfo(np.uint64).max
+        want = np.full(R, np.nan)
+        want[ok] = -np.log(p.astype(np.float64)[idx[ok].astype(np.int64)])
+        assert_close(host(nll), want, "nll gather", abs_floor=1e-6)
+        assert_close(host(nll), oracle.softmax_cat_nll(K, R, p, lab, f64=True), "nll", abs_floor=1e-6)
+
+        dx = empty(K * R, offset=offset)
+        call("anode_gpu_softmax_cat_nll_bwd_packed_f32", K, R, dev(dy, offset), p_d, dev(lab, offset), dx)
+        assert_bit_exact(host(dx), oracle.softmax_cat_nll_bwd(K, R, dy, p, lab), "nll bwd vs fp32")
+        assert_close(host(dx), oracle.softmax_cat_nll_bwd(K, R, dy, p, lab, f64=True), "nll bwd", abs_floor=1e-7)
+        dxa = dev(old, offset)
+        call("anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32", K, R, dev(dy, offset), p_d, dev(lab, offset), dxa)
+        assert_bit_exact(host(dxa), oracle.softmax_cat_nll_bwd(K, R, dy, p, lab, dx_in=old), "nll bwd acc vs fp32")
+
+
+# ---- n-d form ----
+
+ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100, 1, 3), (36, 4, 2), (40, 8, 3),
+             (28, 16, 2), (12, 24, 2), (16, 32, 2), (8, 33, 2), (8, 64, 3), (6, 100, 2), (4, 130, 2), (7, 40, 3)]
+
+
+@pytest.mark.parametrize("P,C,N", ND_SHAPES)
+def test_softmax_nd_all_symbols(oracle, P, C, N):
+    print(f"case P={P} C={C} N={N}", flush=True)
+    g = np.random.default_rng(P * 3 + C)
+    n = P * C * N
+    x = g.standard_normal(n).astype(F32)
+    lab = g.integers(0, C, P * N).astype(np.uint32)
+    lab[g.random(P * N) < 0.05] = 255 if C <= 255 else 0xFFFFFFFF  # ignore-index style labels
+    dy = g.standard_normal(P * N).astype(F32)
+    old = g.standard_normal(n).astype(F32)
+    for offset in (0, 1):
+        p_d = empty(n, offset=offset)
+        call("anode_gpu_softmax_nd_packed_f32", P, C, N, dev(x, offset), p_d)
+        p = host(p_d)
+        assert_close(p, oracle.softmax_nd(P, C, N, x, f64=True), "softmax_nd", abs_floor=1e-30)
+
+        nll = empty(P * N, offset=offset)
+        call("anode_gpu_softmax_nd_cat_nll_packed_f32", P, C, N, p_d, dev(lab, offset), nll)
+        idx = oracle.softmax_nd_cat_gather_index(P, C, N, lab)
+        ok = idx != np.iinfo(np.uint64).max
+        want = np.full(P * N, np.nan)
+        want[ok] = -np.log(p.astype(np.float64)[idx[ok].astype(np.int64)])
+        assert_close(host(nll), want, "nd nll gather", abs_floor=1e-6)
+        assert np.array_equal(np.isnan(host(nll)), lab >= C)
+
+        dx = empty(n, offset=offset)
+        call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dev(dy, offset), p_d, dev(lab, offset), dx)
+        assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "nd bwd vs fp32")
+        assert_close(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, f64=True), "nd bwd", abs_floor=1e-7)
+        dxa = dev(old, offset)
+        call("anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32", P, C, N, dev(dy, offset), p_d,
+             dev(lab, offset), dxa)
+        assert_bit_exact(host(dxa), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, dx_in=old), "nd bwd acc vs fp32")
