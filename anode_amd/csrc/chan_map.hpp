@@ -41,7 +41,7 @@ __device__ inline void lane_set<f32x4>(f32x4 &v, int k, float x) { v[k] = x; }
 template <typename V, int NIN, bool ACC, int UNROLL, typename Op>
 __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
                                                           FastDiv div_c, Op op, const float *a_,
-                                                          const float *b_, float *out_, int nontemporal) {
+                                                          const float *b_, float *out_, int nt) {
   constexpr int L = VecLanes<V>::n;
   const V *a = reinterpret_cast<const V *>(a_);
   const V *b = reinterpret_cast<const V *>(b_);
@@ -55,9 +55,9 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
-        if (NIN >= 1) va[u] = a[g];
-        if (NIN >= 2) vb[u] = b[g];
-        if (ACC) vo[u] = out[g];
+        if (NIN >= 1) va[u] = load_stream(&a[g], nt);
+        if (NIN >= 2) vb[u] = load_stream(&b[g], nt);
+        if (ACC) vo[u] = load_stream(&out[g], nt);
       }
     }
 #pragma unroll
@@ -83,11 +83,7 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
             }
           }
         }
-        if (nontemporal) {
-          __builtin_nontemporal_store(r, &out[g]);
-        } else {
-          out[g] = r;
-        }
+        store_stream(&out[g], r, nt);
       }
     }
   }
@@ -113,10 +109,19 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
   hipStream_t s = as_stream(stream);
   const FastDiv div_s(S), div_c(C);
   const bool vec = aligned16(out) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
+  const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
-    chan_map_kernel<f32x4, NIN, ACC, 4, Op>
-        <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, t.nontemporal);
+    if (t.flat_unroll >= 4) {
+      chan_map_kernel<f32x4, NIN, ACC, 4, Op>
+          <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+    } else if (t.flat_unroll >= 2) {
+      chan_map_kernel<f32x4, NIN, ACC, 2, Op>
+          <<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+    } else {
+      chan_map_kernel<f32x4, NIN, ACC, 1, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+    }
   } else {
     chan_map_kernel<float, NIN, ACC, 4, Op>
         <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, out, 0);

@@ -62,7 +62,7 @@ template <typename Op, typename V>
 __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
-                                                                   double *__restrict__ part) {
+                                                                   double *__restrict__ part, int policy) {
   constexpr int W = VecLanes<V>::n;
   constexpr int U = 4;
   __shared__ double lds[kBlock / kWave];
@@ -92,8 +92,8 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
       for (int u = 0; u < U; ++u) {
         const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
         if (j < LG) {
-          va[u] = pa[j];
-          if (Op::NIN >= 2) vb[u] = pb[j];
+          va[u] = load_stream(&pa[j], policy);
+          if (Op::NIN >= 2) vb[u] = load_stream(&pb[j], policy);
         }
       }
 #pragma unroll
@@ -129,7 +129,7 @@ template <typename Op, typename V>
 __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl, FastDiv div_s, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
-                                                                   double *__restrict__ part) {
+                                                                   double *__restrict__ part, int policy) {
   constexpr int W = VecLanes<V>::n;
   constexpr int G = 16 / W;                       // position groups owned by a thread
   constexpr int STAGES = (Op::NIN >= 2) ? 1 : 2;  // samples loaded before any is consumed
@@ -171,8 +171,8 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
 #pragma unroll
         for (int i = 0; i < G; ++i) {
           if (valid[i]) {
-            va[sg][i] = pa[threadIdx.x + uint32_t(i) * kBlock];
-            if (Op::NIN >= 2) vb[sg][i] = pb[threadIdx.x + uint32_t(i) * kBlock];
+            va[sg][i] = load_stream(&pa[threadIdx.x + uint32_t(i) * kBlock], policy);
+            if (Op::NIN >= 2) vb[sg][i] = load_stream(&pb[threadIdx.x + uint32_t(i) * kBlock], policy);
           }
         }
       }
@@ -261,6 +261,7 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
   const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b));
   const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
   if (Op::NIN < 2) b = a;
+  const int nt = stream_policy(size_t(len) * sizeof(float), tuning().reduce_nontemporal);
 
   ScratchLease lease{nullptr, std::unique_lock<std::mutex>()};
   double *part = nullptr;
@@ -271,15 +272,15 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
   if (pl.whole) {
     const FastDiv div_s(S);
     if (pl.vec) {
-      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part);
+      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part, nt);
     } else {
-      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part);
+      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part, nt);
     }
   } else {
     if (pl.vec) {
-      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part);
+      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part, nt);
     } else {
-      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part);
+      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part, nt);
     }
   }
   note_launch(symbol);

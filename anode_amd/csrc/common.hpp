@@ -70,6 +70,25 @@ struct FastDiv {
 // ---------------------------------------------------------------------------
 #if defined(__HIPCC__)
 
+// Streaming accesses.  Bit 0 of `nt` marks stores, bit 1 marks loads as
+// non-temporal (the `nt` cache policy of global_load/global_store): the data is
+// touched once, so it should not displace reusable lines.
+constexpr int kNtStore = 1, kNtLoad = 2;
+
+template <typename V>
+__device__ inline V load_stream(const V *p, int nt) {
+  return (nt & kNtLoad) ? __builtin_nontemporal_load(p) : *p;
+}
+
+template <typename V>
+__device__ inline void store_stream(V *p, V v, int nt) {
+  if (nt & kNtStore) {
+    __builtin_nontemporal_store(v, p);
+  } else {
+    *p = v;
+  }
+}
+
 template <typename T>
 __device__ inline T wave_sum(T v) {
 #pragma unroll
@@ -124,11 +143,16 @@ int device_cu_count();
 // Tunable launch parameters; defaults are set in runtime.hip and may be
 // changed at run time through anode_gpu_set_tuning().
 struct Tuning {
-  int flat_wg_per_cu;     // resident workgroups per CU targeted by streaming maps
-  int flat_unroll;        // independent 16-byte groups per thread and loop trip
+  int flat_wg_per_cu;     // workgroups per CU of a streaming map; 0 = one trip per workgroup (full grid)
+  int flat_unroll;        // independent 16-byte groups per thread and loop trip (1, 2, 4 or 8)
   int reduce_wg_target;   // workgroups a per-channel reduction aims to launch
-  int nontemporal;        // 1: streaming stores bypass the caches
+  int nontemporal;        // bit 0: non-temporal stores, bit 1: non-temporal loads (streaming maps)
+  int reduce_nontemporal; // bit 1: non-temporal loads in the reductions
+  int nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
 };
+
+// The non-temporal mask to use for an array of `bytes` bytes.
+int stream_policy(size_t bytes, int mask);
 Tuning &tuning();
 
 // Grid size for a grid-stride streaming kernel over `work_items` units of

@@ -81,17 +81,12 @@ ANODE_EXPORT void anode_gpu_discrete_one_hot_3d1_packed_f32(uint32_t dim0, uint3
   const uint32_t len = checked_len(dim0, cat_dim1, dim2, __func__);
   if (len == 0) return;
   hipStream_t s = as_stream(stream);
-  const uint32_t cap = uint32_t(device_cu_count()) * 8u;
   if (dim0 % 4 == 0 && aligned16(x) && aligned16(y)) {
     const uint32_t gps = dim0 / 4, total = gps * dim2;
-    uint32_t blocks = (total + kBlock - 1) / kBlock;
-    if (blocks > cap) blocks = cap;
-    one_hot_kernel<4><<<blocks, kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(gps), x, y);
+    one_hot_kernel<4><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(gps), x, y);
   } else {
     const uint32_t total = dim0 * dim2;
-    uint32_t blocks = (total + kBlock - 1) / kBlock;
-    if (blocks > cap) blocks = cap;
-    one_hot_kernel<1><<<blocks, kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(dim0), x, y);
+    one_hot_kernel<1><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(dim0), x, y);
   }
   note_launch(__func__);
 }

@@ -73,21 +73,12 @@ __device__ inline f32x4 apply_vec(const Op &op, f32x4 a, f32x4 b) {
   return r;
 }
 
-template <typename V>
-__device__ inline void store_vec(V *p, V v, bool nontemporal) {
-  if (nontemporal) {
-    __builtin_nontemporal_store(v, p);
-  } else {
-    *p = v;
-  }
-}
-
 // n_groups groups of Lanes<V>::n elements, then `tail` single elements that
 // start at element n_groups * Lanes<V>::n (handled by workgroup 0).
 template <typename V, int NIN, int UNROLL, typename Op>
 __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uint32_t tail, Op op,
                                                           const float *a_, const float *b_,
-                                                          float *out_, int nontemporal) {
+                                                          float *out_, int nt) {
   // no __restrict__: out_ may alias a_ or b_ at equal index
   const V *a = reinterpret_cast<const V *>(a_);
   const V *b = reinterpret_cast<const V *>(b_);
@@ -100,14 +91,14 @@ __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uin
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
-        va[u] = a[g];
-        vb[u] = (NIN == 2) ? b[g] : va[u];
+        va[u] = load_stream(&a[g], nt);
+        vb[u] = (NIN == 2) ? load_stream(&b[g], nt) : va[u];
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) store_vec(&out[g], apply_vec(op, va[u], vb[u]), nontemporal != 0);
+      if (g < n_groups) store_stream(&out[g], apply_vec(op, va[u], vb[u]), nt);
     }
   }
   if (blockIdx.x == 0 && threadIdx.x < tail) {
@@ -125,14 +116,17 @@ void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, co
   const Tuning &t = tuning();
   const bool vec = aligned16(a) && aligned16(out) && (NIN == 1 || aligned16(b));
   hipStream_t s = as_stream(stream);
+  const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
     if (t.flat_unroll >= 8) {
-      flat_map_kernel<f32x4, NIN, 8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+      flat_map_kernel<f32x4, NIN, 8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, a, b, out, nt);
     } else if (t.flat_unroll >= 4) {
-      flat_map_kernel<f32x4, NIN, 4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+      flat_map_kernel<f32x4, NIN, 4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, a, b, out, nt);
+    } else if (t.flat_unroll >= 2) {
+      flat_map_kernel<f32x4, NIN, 2, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, a, b, out, nt);
     } else {
-      flat_map_kernel<f32x4, NIN, 2, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, a, b, out, t.nontemporal);
+      flat_map_kernel<f32x4, NIN, 1, Op><<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out, nt);
     }
   } else {
     flat_map_kernel<float, NIN, 4, Op><<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, op, a, b, out, 0);
@@ -161,7 +155,7 @@ template <int UNROLL, typename Op>
 __global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, uint32_t tail, Op op,
                                                             const uint8_t *__restrict__ x,
                                                             typename Op::out_t *__restrict__ y,
-                                                            int nontemporal) {
+                                                            int nt) {
   typedef typename Op::out4_t O4;
   const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
   O4 *y4 = reinterpret_cast<O4 *>(y);
@@ -172,7 +166,7 @@ __global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, u
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) w[u] = x4[g];
+      if (g < n_groups) w[u] = load_stream(&x4[g], nt);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -183,7 +177,7 @@ __global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, u
         r.y = op((w[u] >> 8) & 0xffu);
         r.z = op((w[u] >> 16) & 0xffu);
         r.w = op(w[u] >> 24);
-        store_vec(&y4[g], r, nontemporal != 0);
+        store_stream(&y4[g], r, nt);
       }
     }
   }
@@ -209,10 +203,16 @@ void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, 
   hipStream_t s = as_stream(stream);
   if (aligned4(x) && aligned16(y)) {
     const uint32_t groups = len / 4, tail = len % 4;
+    // the policy looks at the output, which is four times the input
+    const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
     if (t.flat_unroll >= 8) {
-      widen_u8x4_kernel<8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, x, y, t.nontemporal);
+      widen_u8x4_kernel<8, Op><<<stream_grid(groups, 8), kBlock, 0, s>>>(groups, tail, op, x, y, nt);
+    } else if (t.flat_unroll >= 4) {
+      widen_u8x4_kernel<4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, x, y, nt);
+    } else if (t.flat_unroll >= 2) {
+      widen_u8x4_kernel<2, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, x, y, nt);
     } else {
-      widen_u8x4_kernel<4, Op><<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, op, x, y, t.nontemporal);
+      widen_u8x4_kernel<1, Op><<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, x, y, nt);
     }
   } else {
     widen_u8_scalar_kernel<Op><<<stream_grid(len, 1), kBlock, 0, s>>>(len, op, x, y);

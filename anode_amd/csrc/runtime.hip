@@ -26,10 +26,12 @@ std::mutex g_scratch_mutex;
 std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch;
 
 Tuning g_tuning = {
-    /*flat_wg_per_cu=*/8,
-    /*flat_unroll=*/4,
+    /*flat_wg_per_cu=*/0,
+    /*flat_unroll=*/1,
     /*reduce_wg_target=*/2048,
     /*nontemporal=*/0,
+    /*reduce_nontemporal=*/0,
+    /*nt_min_bytes=*/192 << 20,
 };
 
 }  // namespace
@@ -51,10 +53,16 @@ Tuning &tuning() { return g_tuning; }
 uint32_t stream_grid(uint64_t work_items, int items_per_thread) {
   const uint64_t per_block = uint64_t(kBlock) * uint64_t(items_per_thread > 0 ? items_per_thread : 1);
   uint64_t blocks = (work_items + per_block - 1) / per_block;
-  const uint64_t cap = uint64_t(device_cu_count()) * uint64_t(g_tuning.flat_wg_per_cu);
-  if (blocks > cap) blocks = cap;
+  if (g_tuning.flat_wg_per_cu > 0) {
+    const uint64_t cap = uint64_t(device_cu_count()) * uint64_t(g_tuning.flat_wg_per_cu);
+    if (blocks > cap) blocks = cap;
+  }
   if (blocks < 1) blocks = 1;
   return uint32_t(blocks);
+}
+
+int stream_policy(size_t bytes, int mask) {
+  return bytes >= size_t(g_tuning.nt_min_bytes > 0 ? g_tuning.nt_min_bytes : 0) ? mask : 0;
 }
 
 void require_pow2_block(const KernelConfig *cfg, const char *symbol) {
@@ -207,7 +215,8 @@ ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int 
 // the kernels compute it.
 ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return anode::FastDiv(d).div(n); }
 
-// Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal.
+// Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal,
+// 4 reduce_nontemporal, 5 nt_min_bytes.
 // Returns the previous value, or -1 for an unknown knob.  A negative value
 // only reads.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
@@ -218,6 +227,8 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 1: slot = &t.flat_unroll; break;
     case 2: slot = &t.reduce_wg_target; break;
     case 3: slot = &t.nontemporal; break;
+    case 4: slot = &t.reduce_nontemporal; break;
+    case 5: slot = &t.nt_min_bytes; break;
     default: return -1;
   }
   const int old = *slot;

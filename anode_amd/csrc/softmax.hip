@@ -357,12 +357,8 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W) {
   return pg;
 }
 
-uint32_t pixel_blocks(uint32_t total_groups) {
-  const uint32_t cap = uint32_t(device_cu_count()) * 8u;
-  uint32_t blocks = (total_groups + kBlock - 1) / kBlock;
-  if (blocks > cap) blocks = cap;
-  return blocks ? blocks : 1;
-}
+// one pixel group per thread: the hardware dispatcher walks the array in order
+uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
 template <typename V>
 void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, hipStream_t s) {
