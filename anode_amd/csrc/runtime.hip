@@ -28,7 +28,7 @@ std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch;
 Tuning g_tuning = {
     /*flat_wg_per_cu=*/0,
     /*flat_unroll=*/1,
-    /*reduce_wg_target=*/2048,
+    /*reduce_wg_target=*/8192,
     /*nontemporal=*/0,
     /*reduce_nontemporal=*/0,
     /*nt_min_bytes=*/192 << 20,

@@ -35,6 +35,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated group names to run (default: all)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="add one plain copy of a known size to the step (scale for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -45,7 +47,7 @@ class Launch:
         self.group, self.symbol, self.args, self.alg_bytes, self.elements = group, symbol, args, alg_bytes, elements
 
 
-def build_workload(torch, only):
+def build_workload(torch, only, copy_calibration=False):
     """All device buffers and the launch list of one step."""
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
@@ -65,6 +67,11 @@ def build_workload(torch, only):
 
     def want(group):
         return not only or group in only
+
+    if copy_calibration:
+        n = 64 * 1024 * 1024  # 256 MiB in, 256 MiB out
+        src, dst = randn(n), empty(n)
+        launches.append(Launch("copy_calibration", "anode_gpu_copy_flat_map_f32", (n, src, dst), 8 * n, n))
 
     # ---- config 1: u8 image batch [256,3,224,224] -> f32 / u32 -------------------
     if want("cast_cfg1"):
@@ -211,7 +218,7 @@ def main():
         sys.exit(3)
     torch.cuda.set_device(0)
     only = set(filter(None, args.only.split(",")))
-    launches = build_workload(torch, only)
+    launches = build_workload(torch, only, args.copy_calibration)
     torch.cuda.synchronize()
 
     def run_step(wrap_symbol=None, events=None):
