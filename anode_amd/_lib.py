@@ -29,10 +29,11 @@ _SCALARS = {
     "uint32_t": ctypes.c_uint32,
     "int": ctypes.c_int,
     "float": ctypes.c_float,
+    "size_t": ctypes.c_size_t,
     "void": None,
 }
 
-_DECL = re.compile(r"^\s*(void|int|uint32_t)\s+(anode_gpu_\w+)\s*\(([^;]*)\)\s*;", re.M)
+_DECL = re.compile(r"^\s*(void|int|uint32_t|size_t)\s+(anode_(?:gpu|host)_\w+)\s*\(([^;]*)\)\s*;", re.M)
 
 
 def _ctype_of(param: str):

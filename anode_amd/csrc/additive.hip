@@ -1,0 +1,514 @@
+// Entry points that have no kernel in the reference but sit directly on either
+// side of the hot path: the inverse of dequantize, the per-channel affine and
+// channel sums that the reference only declares (commented out in
+// routines_gpu/lib.h:195-249, 406-430), single-pass batch statistics, fused
+// batch-norm forward/backward, running averages and arg-max.  They reuse the
+// map / reduce templates of the reference ABI kernels.
+#include "chan_map.hpp"
+#include "chan_reduce.hpp"
+#include "common.hpp"
+
+#include <cmath>
+
+namespace anode {
+namespace {
+
+struct Empty {};
+
+// ---------------------------------------------------------------------------
+// f32 -> u8 quantisation: q = clamp(rint((x - lo) / scale), 0, 255), NaN -> 0,
+// scale = (hi - lo) / 255; rint rounds half to even.  Inverse of dequantize.
+// ---------------------------------------------------------------------------
+__device__ inline uint32_t quantize_one(float x, float lo, float scale) {
+  float q = rintf((x - lo) / scale);
+  q = (q >= 0.0f) ? q : 0.0f;  // also catches NaN
+  q = (q > 255.0f) ? 255.0f : q;
+  return uint32_t(q);
+}
+
+__global__ __launch_bounds__(kBlock) void quantize_u8x4_kernel(uint32_t n_groups, uint32_t tail, float lo,
+                                                               float scale, const float *__restrict__ x,
+                                                               uint8_t *__restrict__ y) {
+  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+  uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < n_groups; g += stride) {
+    const f32x4 v = x4[g];
+    y4[g] = quantize_one(v.x, lo, scale) | (quantize_one(v.y, lo, scale) << 8) |
+            (quantize_one(v.z, lo, scale) << 16) | (quantize_one(v.w, lo, scale) << 24);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * 4u + threadIdx.x;
+    y[i] = uint8_t(quantize_one(x[i], lo, scale));
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void quantize_u8_scalar_kernel(uint32_t len, float lo, float scale,
+                                                                    const float *__restrict__ x,
+                                                                    uint8_t *__restrict__ y) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = uint8_t(quantize_one(x[i], lo, scale));
+}
+
+// ---------------------------------------------------------------------------
+// per-channel affine maps
+// ---------------------------------------------------------------------------
+
+// y = lx[b] * rx  /  y = fma(lx[b], rx, shift[b])
+struct BcastMultMap {
+  const float *lx;
+  struct Param { float l; };
+  __device__ Param load(uint32_t c) const { return Param{lx[c]}; }
+  __device__ float value(const Param &p, float r, float, uint32_t) const { return p.l * r; }
+  __device__ float accum(const Param &p, float r, float, uint32_t, float old) const { return fmaf(p.l, r, old); }
+};
+struct BcastMultAddMap {
+  const float *lx, *shift;
+  struct Param { float l, s; };
+  __device__ Param load(uint32_t c) const { return Param{lx[c], shift[c]}; }
+  __device__ float value(const Param &p, float r, float, uint32_t) const { return fmaf(p.l, r, p.s); }
+  __device__ float accum(const Param &p, float r, float, uint32_t, float old) const { return old + fmaf(p.l, r, p.s); }
+};
+// y = fma(lx, rx, shift), all three per element
+struct FlatMultAddMap {
+  typedef Empty Param;
+  __device__ Param load(uint32_t) const { return Param{}; }
+  __device__ float value3(const Param &, float l, float r, float s, uint32_t) const { return fmaf(l, r, s); }
+  __device__ float accum3(const Param &, float l, float r, float s, uint32_t, float old) const {
+    return old + fmaf(l, r, s);
+  }
+};
+struct FlatMultMap {
+  typedef Empty Param;
+  __device__ Param load(uint32_t) const { return Param{}; }
+  __device__ float value(const Param &, float l, float r, uint32_t) const { return l * r; }
+  __device__ float accum(const Param &, float l, float r, uint32_t, float old) const { return fmaf(l, r, old); }
+};
+
+// u8 codes -> per-channel affine f32: y = fma(scale[b], float(q), shift[b]).
+// Each lane loads one dword (4 codes) and stores 16 bytes; the channel of the
+// group's first code is found by exact division, then advanced incrementally.
+__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t n_groups, uint32_t tail,
+                                                                       FastDiv div_s, FastDiv div_c,
+                                                                       const float *__restrict__ scale,
+                                                                       const float *__restrict__ shift,
+                                                                       const uint8_t *__restrict__ x,
+                                                                       float *__restrict__ y) {
+  const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
+  f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
+  const uint32_t S = div_s.d, C = div_c.d;
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < n_groups; g += stride) {
+    const uint32_t w = x4[g];
+    uint32_t q, s;
+    div_s.divmod(g * 4u, q, s);
+    uint32_t c = q - div_c.div(q) * C;
+    float a = scale[c], b = shift[c];
+    f32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      r[k] = fmaf(a, float((w >> (8 * k)) & 0xffu), b);
+      if (k < 3 && ++s == S) {
+        s = 0;
+        c = (c + 1 == C) ? 0 : c + 1;
+        a = scale[c];
+        b = shift[c];
+      }
+    }
+    y4[g] = r;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * 4u + threadIdx.x;
+    const uint32_t q = div_s.div(i);
+    const uint32_t c = q - div_c.div(q) * C;
+    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8_scalar_kernel(uint32_t len, FastDiv div_s,
+                                                                            FastDiv div_c,
+                                                                            const float *__restrict__ scale,
+                                                                            const float *__restrict__ shift,
+                                                                            const uint8_t *__restrict__ x,
+                                                                            float *__restrict__ y) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) {
+    const uint32_t q = div_s.div(i);
+    const uint32_t c = q - div_c.div(q) * div_c.d;
+    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// per-channel sums and single-pass statistics
+// ---------------------------------------------------------------------------
+
+struct SumReduce {
+  static constexpr int NIN = 1, NACC = 1;
+  typedef Empty Param;
+  float *y;
+  bool square;
+  __device__ Param load(uint32_t) const { return Param{}; }
+  __device__ void term(const Param &, float a, float, double &s0, double &, double &) const {
+    const double d = double(a);
+    s0 = square ? fma(d, d, s0) : s0 + d;
+  }
+  __device__ void finalize(uint32_t c, double s0, double, double) const { y[c] = float(s0); }
+};
+
+// mean and biased variance + eps in one pass over x.  Sums are taken about a
+// per-channel shift K (the channel's first element), which keeps
+// sum (x-K)^2 - (sum (x-K))^2 / n well conditioned for any offset of the data.
+struct MeanVarReduce {
+  static constexpr int NIN = 1, NACC = 2;
+  typedef double Param;
+  const float *x;
+  float *mean, *var;
+  uint32_t S;
+  double n, eps;
+  __device__ Param load(uint32_t c) const { return double(x[size_t(c) * S]); }
+  __device__ void term(const Param &k, float a, float, double &s0, double &s1, double &) const {
+    const double d = double(a) - k;
+    s0 += d;
+    s1 = fma(d, d, s1);
+  }
+  __device__ void finalize(uint32_t c, double s0, double s1, double) const {
+    const double k = double(x[size_t(c) * S]);
+    mean[c] = float(k + s0 / n);
+    var[c] = float((s1 - s0 * s0 / n) / n + eps);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// fused batch-norm forward maps
+// ---------------------------------------------------------------------------
+
+// y = relu_by_multiply((x - m) * rs): batch_norm followed by positive_clip in one pass
+struct NormPositiveClipMap {
+  const float *mean, *var;
+  struct Param { float m, rs; };
+  __device__ Param load(uint32_t c) const { return Param{mean[c], 1.0f / sqrtf(var[c])}; }
+  __device__ float value(const Param &p, float x, float, uint32_t) const {
+    const float t = (x - p.m) * p.rs;
+    return t * float(t > 0.0f);
+  }
+  __device__ float accum(const Param &p, float x, float, uint32_t s, float old) const { return old + value(p, x, 0.0f, s); }
+};
+
+// y = fma((x - m) * rs, gamma[c], beta[c]): batch_norm followed by the per-channel affine
+struct NormAffineMap {
+  const float *mean, *var, *gamma, *beta;
+  struct Param { float m, rs, g, b; };
+  __device__ Param load(uint32_t c) const { return Param{mean[c], 1.0f / sqrtf(var[c]), gamma[c], beta[c]}; }
+  __device__ float value(const Param &p, float x, float, uint32_t) const { return fmaf((x - p.m) * p.rs, p.g, p.b); }
+  __device__ float accum(const Param &p, float x, float, uint32_t s, float old) const { return old + value(p, x, 0.0f, s); }
+};
+
+// ---------------------------------------------------------------------------
+// fused batch-norm backward: one reduction pass over (dy, x), one map pass
+// ---------------------------------------------------------------------------
+
+// dvar = sum dy (x-m) * (-0.5 rs / v);  dmean = -rs sum dy + (sum (x-m)) (-2 dvar) / n.
+// With a mask array (the ReLU output) dy is first multiplied by float(mask > 0).
+template <bool MASKED>
+struct NormBwdFusedReduce {
+  static constexpr int NIN = MASKED ? 3 : 2, NACC = 3;  // a = dy, b = x, c = mask
+  typedef double Param;
+  const float *mean, *var;
+  float *dmean, *dvar;
+  double n;
+  __device__ Param load(uint32_t c) const { return double(mean[c]); }
+  __device__ void term(const Param &m, float dy, float x, double &s0, double &s1, double &s2) const {
+    const double d = double(x) - m;
+    s0 += double(dy);
+    s1 = fma(double(dy), d, s1);
+    s2 += d;
+  }
+  __device__ void term3(const Param &m, float dy, float x, float mask, double &s0, double &s1, double &s2) const {
+    term(m, dy * float(mask > 0.0f), x, s0, s1, s2);
+  }
+  __device__ void finalize(uint32_t c, double s0, double s1, double s2) const {
+    const double v = double(var[c]);
+    const double rs = 1.0 / sqrt(v);
+    const double dv = s1 * (-0.5 * rs / v);
+    dvar[c] = float(dv);
+    dmean[c] = float(-rs * s0 + s2 * (-2.0 * dv) / n);
+  }
+};
+
+// dx (=|+=) dy*rs + dvar*(x-m)*2/n + dmean/n, each term in the arithmetic of the
+// three separate launches it replaces and added in their order
+template <bool MASKED>
+struct NormBwdFusedMap {
+  const float *mean, *var, *dmean, *dvar;
+  float norm;
+  struct Param { float m, rs, dv, dm; };
+  __device__ Param load(uint32_t c) const {
+    return Param{mean[c], 1.0f / sqrtf(var[c]), dvar[c], dmean[c] / norm};
+  }
+  __device__ float core(const Param &p, float dy, float x) const {
+    return (dy * p.rs + p.dv * (x - p.m) * 2.0f / norm) + p.dm;
+  }
+  __device__ float value(const Param &p, float dy, float x, uint32_t) const { return core(p, dy, x); }
+  __device__ float accum(const Param &p, float dy, float x, uint32_t, float old) const {
+    return ((fmaf(dy, p.rs, old)) + p.dv * (x - p.m) * 2.0f / norm) + p.dm;
+  }
+  __device__ float value3(const Param &p, float dy, float x, float mask, uint32_t) const {
+    return core(p, dy * float(mask > 0.0f), x);
+  }
+  __device__ float accum3(const Param &p, float dy, float x, float mask, uint32_t s, float old) const {
+    return accum(p, dy * float(mask > 0.0f), x, s, old);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// running average, arg-max
+// ---------------------------------------------------------------------------
+
+// y <- y + rate * (x - y)
+struct OnlineAverageMap {
+  float rate;
+  __device__ float operator()(float x, float y) const { return fmaf(rate, x - y, y); }
+};
+
+__global__ __launch_bounds__(kBlock) void online_average_kernel(uint32_t len, float rate,
+                                                                const float *__restrict__ x, float *y) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = fmaf(rate, x[i] - y[i], y[i]);
+}
+
+// First index of the strict maximum of each row of a [K (fastest), R] array;
+// NaN never wins; a row without any value above -inf gives 0.  One wave per row.
+__global__ __launch_bounds__(kBlock) void arg_max_rows_kernel(uint32_t K, uint32_t R, const float *__restrict__ x,
+                                                              uint32_t *__restrict__ out) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
+  const uint32_t n_waves = gridDim.x * (kBlock / kWave);
+  for (uint32_t r = wave; r < R; r += n_waves) {
+    const float *xr = x + size_t(r) * K;
+    float top = -__builtin_huge_valf();
+    uint32_t idx = 0xffffffffu;  // nothing above -inf seen yet
+    for (uint32_t k = lane; k < K; k += kWave) {
+      const float v = xr[k];
+      if (v > top) {
+        top = v;
+        idx = k;
+      }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      const float t2 = __shfl_xor(top, off, kWave);
+      const uint32_t i2 = __shfl_xor(idx, off, kWave);
+      if (t2 > top || (t2 == top && i2 < idx)) {
+        top = t2;
+        idx = i2;
+      }
+    }
+    if (lane == 0) out[r] = (idx == 0xffffffffu) ? 0u : idx;
+  }
+}
+
+void launch_quantize(const char *symbol, uint32_t len, float lo, float hi, const float *x, uint8_t *y,
+                     CUstream_st *stream) {
+  if (len == 0) return;
+  const float scale = (hi - lo) / 255.0f;
+  hipStream_t s = as_stream(stream);
+  if (aligned16(x) && aligned4(y)) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    quantize_u8x4_kernel<<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, lo, scale, x, y);
+  } else {
+    quantize_u8_scalar_kernel<<<stream_grid(len, 1), kBlock, 0, s>>>(len, lo, scale, x, y);
+  }
+  note_launch(symbol);
+}
+
+}  // namespace
+}  // namespace anode
+
+using namespace anode;
+
+ANODE_EXPORT void anode_gpu_quantize_u8_packed_f32(uint32_t len, float lo, float hi, const float *x, uint8_t *y,
+                                                   const KernelConfig *, CUstream_st *stream) {
+  launch_quantize(__func__, len, lo, hi, x, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_bcast_flat_mult_I1b_I2ab_Oab_packed_f32(uint32_t inner_dim, uint32_t bcast_dim,
+                                                                    const float *lx, const float *rx, float *y,
+                                                                    const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, inner_dim, bcast_dim, 1, BcastMultMap{lx}, rx, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_bcast_flat_mult_add_I1b_I2ab_Oab_packed_f32(uint32_t inner_dim, uint32_t bcast_dim,
+                                                                        const float *lx, const float *rx,
+                                                                        const float *shift, float *y,
+                                                                        const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, inner_dim, bcast_dim, 1, BcastMultAddMap{lx, shift}, rx, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_bcast_flat_mult_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim,
+                                                                      uint32_t outer_dim, const float *lx,
+                                                                      const float *rx, float *y,
+                                                                      const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, inner_dim, bcast_dim, outer_dim, BcastMultMap{lx}, rx, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_bcast_flat_mult_add_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim,
+                                                                          uint32_t outer_dim, const float *lx,
+                                                                          const float *rx, const float *shift,
+                                                                          float *y, const KernelConfig *,
+                                                                          CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, inner_dim, bcast_dim, outer_dim, BcastMultAddMap{lx, shift}, rx, nullptr, y,
+                            stream);
+}
+
+ANODE_EXPORT void anode_gpu_flat_mult_f32(uint32_t len, const float *lx, const float *rx, float *y,
+                                          const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<2, false>(__func__, len, 1, 1, FlatMultMap{}, lx, rx, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_flat_mult_add_f32(uint32_t len, const float *lx, const float *rx, const float *shift,
+                                              float *y, const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<3, false>(__func__, len, 1, 1, FlatMultAddMap{}, lx, rx, y, stream, shift);
+}
+
+ANODE_EXPORT void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim,
+                                                                          uint32_t outer_dim, const float *scale,
+                                                                          const float *shift, const uint8_t *x,
+                                                                          float *y, const KernelConfig *,
+                                                                          CUstream_st *stream) {
+  const uint32_t len = checked_len(inner_dim, bcast_dim, outer_dim, __func__);
+  if (len == 0) return;
+  hipStream_t s = as_stream(stream);
+  const FastDiv div_s(inner_dim), div_c(bcast_dim);
+  if (aligned4(x) && aligned16(y)) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    bcast_dequantize_u8x4_kernel<<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, scale, shift, x, y);
+  } else {
+    bcast_dequantize_u8_scalar_kernel<<<stream_grid(len, 1), kBlock, 0, s>>>(len, div_s, div_c, scale, shift, x, y);
+  }
+  note_launch(__func__);
+}
+
+ANODE_EXPORT void anode_gpu_sum_Iab_Ob_packed_deterministic_f32(uint32_t reduce_dim, uint32_t outer_dim,
+                                                                const float *x, float *y, const KernelConfig *,
+                                                                CUstream_st *stream) {
+  launch_chan_reduce(__func__, reduce_dim, outer_dim, 1, SumReduce{y, false}, x, nullptr, stream);
+}
+
+ANODE_EXPORT void anode_gpu_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, uint32_t mid_dim,
+                                                                 uint32_t reduce_outer_dim, const float *x, float *y,
+                                                                 const KernelConfig *, CUstream_st *stream) {
+  launch_chan_reduce(__func__, reduce_inner_dim, mid_dim, reduce_outer_dim, SumReduce{y, false}, x, nullptr, stream);
+}
+
+ANODE_EXPORT void anode_gpu_square_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, uint32_t mid_dim,
+                                                                        uint32_t reduce_outer_dim, const float *x,
+                                                                        float *y, const KernelConfig *,
+                                                                        CUstream_st *stream) {
+  launch_chan_reduce(__func__, reduce_inner_dim, mid_dim, reduce_outer_dim, SumReduce{y, true}, x, nullptr, stream);
+}
+
+ANODE_EXPORT void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon,
+                                                          const float *x, float *mean, float *var,
+                                                          const KernelConfig *, CUstream_st *stream) {
+  launch_chan_reduce(__func__, dim0, dim1, dim2,
+                     MeanVarReduce{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)}, x, nullptr, stream);
+}
+
+ANODE_EXPORT void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                                    const float *x, const float *mean,
+                                                                    const float *var, float *y, const KernelConfig *,
+                                                                    CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, dim0, dim1, dim2, NormPositiveClipMap{mean, var}, x, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_batch_norm_affine_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                             const float *x, const float *mean, const float *var,
+                                                             const float *gamma, const float *beta, float *y,
+                                                             const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<1, false>(__func__, dim0, dim1, dim2, NormAffineMap{mean, var, gamma, beta}, x, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_batch_norm_bwd_reduce_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                                 const float *dy, const float *x, const float *mean,
+                                                                 const float *var, const float *mask, float *dmean,
+                                                                 float *dvar, const KernelConfig *,
+                                                                 CUstream_st *stream) {
+  const double n = double(dim0) * double(dim2);
+  if (mask) {
+    launch_chan_reduce(__func__, dim0, dim1, dim2, NormBwdFusedReduce<true>{mean, var, dmean, dvar, n}, dy, x, stream, mask);
+  } else {
+    launch_chan_reduce(__func__, dim0, dim1, dim2, NormBwdFusedReduce<false>{mean, var, dmean, dvar, n}, dy, x, stream);
+  }
+}
+
+static void bwd_apply(const char *symbol, bool accumulate, uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                      const float *dy, const float *x, const float *mean, const float *var, const float *dmean,
+                      const float *dvar, const float *mask, float *dx, CUstream_st *stream) {
+  const float norm = float(dim0) * float(dim2);
+  if (mask) {
+    const NormBwdFusedMap<true> op{mean, var, dmean, dvar, norm};
+    if (accumulate) {
+      launch_chan_map<3, true>(symbol, dim0, dim1, dim2, op, dy, x, dx, stream, mask);
+    } else {
+      launch_chan_map<3, false>(symbol, dim0, dim1, dim2, op, dy, x, dx, stream, mask);
+    }
+  } else {
+    const NormBwdFusedMap<false> op{mean, var, dmean, dvar, norm};
+    if (accumulate) {
+      launch_chan_map<2, true>(symbol, dim0, dim1, dim2, op, dy, x, dx, stream);
+    } else {
+      launch_chan_map<2, false>(symbol, dim0, dim1, dim2, op, dy, x, dx, stream);
+    }
+  }
+}
+
+ANODE_EXPORT void anode_gpu_batch_norm_bwd_apply_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                                const float *dy, const float *x, const float *mean,
+                                                                const float *var, const float *dmean,
+                                                                const float *dvar, const float *mask, float *dx,
+                                                                const KernelConfig *, CUstream_st *stream) {
+  bwd_apply(__func__, false, dim0, dim1, dim2, dy, x, mean, var, dmean, dvar, mask, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_batch_norm_bwd_apply_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1,
+                                                                           uint32_t dim2, const float *dy,
+                                                                           const float *x, const float *mean,
+                                                                           const float *var, const float *dmean,
+                                                                           const float *dvar, const float *mask,
+                                                                           float *dx, const KernelConfig *,
+                                                                           CUstream_st *stream) {
+  bwd_apply(__func__, true, dim0, dim1, dim2, dy, x, mean, var, dmean, dvar, mask, dx, stream);
+}
+
+ANODE_EXPORT void anode_gpu_online_average_packed_f32(uint32_t len, float rate, const float *x, float *y,
+                                                      const KernelConfig *, CUstream_st *stream) {
+  if (len == 0) return;
+  online_average_kernel<<<stream_grid(len, 1), kBlock, 0, as_stream(stream)>>>(len, rate, x, y);
+  note_launch(__func__);
+}
+
+ANODE_EXPORT void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, const float *x, uint32_t *index,
+                                               const KernelConfig *, CUstream_st *stream) {
+  (void)checked_len(dim0, dim1, 1, __func__);
+  if (dim1 == 0) return;
+  const uint32_t waves_per_block = kBlock / kWave;
+  uint32_t blocks = (dim1 + waves_per_block - 1) / waves_per_block;
+  const uint32_t cap = uint32_t(device_cu_count()) * 8u;
+  if (blocks > cap) blocks = cap;
+  arg_max_rows_kernel<<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
+  note_launch(__func__);
+}
+
+// The host rule of src/utils/mod.rs:31-41, for callers that keep logits on the host.
+ANODE_EXPORT size_t anode_host_arg_max_f32(const float *xs, size_t len) {
+  float top_x = -__builtin_huge_valf();
+  size_t top_k = 0;
+  for (size_t k = 0; k < len; ++k) {
+    if (xs[k] > top_x) {
+      top_x = xs[k];
+      top_k = k;
+    }
+  }
+  return top_k;
+}

@@ -30,8 +30,8 @@ struct MeanReduce {
   float *mean;
   double n;
   __device__ Param load(uint32_t) const { return Param{}; }
-  __device__ void term(const Param &, float a, float, double &s0, double &) const { s0 += double(a); }
-  __device__ void finalize(uint32_t c, double s0, double) const { mean[c] = float(s0 / n); }
+  __device__ void term(const Param &, float a, float, double &s0, double &, double &) const { s0 += double(a); }
+  __device__ void finalize(uint32_t c, double s0, double, double) const { mean[c] = float(s0 / n); }
 };
 
 // batch_norm.cu:125-163   var[c] = sum (x - mean[c])^2 / n + eps
@@ -42,11 +42,11 @@ struct VarReduce {
   float *var;
   double n, eps;
   __device__ Param load(uint32_t c) const { return double(mean[c]); }
-  __device__ void term(const Param &m, float a, float, double &s0, double &) const {
+  __device__ void term(const Param &m, float a, float, double &s0, double &, double &) const {
     const double d = double(a) - m;
     s0 = fma(d, d, s0);
   }
-  __device__ void finalize(uint32_t c, double s0, double) const { var[c] = float(s0 / n + eps); }
+  __device__ void finalize(uint32_t c, double s0, double, double) const { var[c] = float(s0 / n + eps); }
 };
 
 // batch_norm.cu:240-280   dmean[c] (=|+=) (sum (x - mean[c]) * (-2 dvar[c])) / n
@@ -58,8 +58,8 @@ struct VarBwdMeanReduce {
   double n;
   bool accumulate;
   __device__ Param load(uint32_t c) const { return double(mean[c]); }
-  __device__ void term(const Param &m, float a, float, double &s0, double &) const { s0 += double(a) - m; }
-  __device__ void finalize(uint32_t c, double s0, double) const {
+  __device__ void term(const Param &m, float a, float, double &s0, double &, double &) const { s0 += double(a) - m; }
+  __device__ void finalize(uint32_t c, double s0, double, double) const {
     write_out(dmean, c, s0 * (-2.0 * double(dvar[c])) / n, accumulate);
   }
 };
@@ -72,8 +72,8 @@ struct NormBwdMeanReduce {
   float *dmean;
   bool accumulate;
   __device__ Param load(uint32_t) const { return Param{}; }
-  __device__ void term(const Param &, float a, float, double &s0, double &) const { s0 += double(a); }
-  __device__ void finalize(uint32_t c, double s0, double) const {
+  __device__ void term(const Param &, float a, float, double &s0, double &, double &) const { s0 += double(a); }
+  __device__ void finalize(uint32_t c, double s0, double, double) const {
     write_out(dmean, c, -s0 / sqrt(double(var[c])), accumulate);
   }
 };
@@ -86,10 +86,10 @@ struct NormBwdVarReduce {
   float *dvar;
   bool accumulate;
   __device__ Param load(uint32_t c) const { return double(mean[c]); }
-  __device__ void term(const Param &m, float a, float b, double &s0, double &) const {
+  __device__ void term(const Param &m, float a, float b, double &s0, double &, double &) const {
     s0 = fma(double(a), double(b) - m, s0);
   }
-  __device__ void finalize(uint32_t c, double s0, double) const {
+  __device__ void finalize(uint32_t c, double s0, double, double) const {
     const double v = double(var[c]);
     write_out(dvar, c, s0 * (-0.5 / (sqrt(v) * v)), accumulate);
   }
@@ -103,10 +103,10 @@ struct NormBwdVarV2Reduce {
   float *dvar;
   bool accumulate;
   __device__ Param load(uint32_t) const { return Param{}; }
-  __device__ void term(const Param &, float a, float b, double &s0, double &) const {
+  __device__ void term(const Param &, float a, float b, double &s0, double &, double &) const {
     s0 = fma(double(a), double(b), s0);
   }
-  __device__ void finalize(uint32_t c, double s0, double) const {
+  __device__ void finalize(uint32_t c, double s0, double, double) const {
     write_out(dvar, c, s0 * (-0.5 / double(var[c])), accumulate);
   }
 };

@@ -19,7 +19,8 @@ namespace anode {
 //   __device__ Param load(uint32_t c) const;
 //   __device__ float value(const Param&, float a, float b, uint32_t s) const;
 //   __device__ float accum(const Param&, float a, float b, uint32_t s, float old) const;
-// where s is the element's position inside its channel run.
+// where s is the element's position inside its channel run.  Ops with a third
+// element input (NIN == 3) define value3/accum3 taking (a, b, c) instead.
 template <typename V> struct VecLanes;
 template <> struct VecLanes<float> { static constexpr int n = 1; };
 template <> struct VecLanes<f32x4> { static constexpr int n = 4; };
@@ -38,25 +39,36 @@ __device__ inline void lane_set<float>(float &v, int, float x) { v = x; }
 template <>
 __device__ inline void lane_set<f32x4>(f32x4 &v, int k, float x) { v[k] = x; }
 
+template <int NIN, bool ACC, typename Op, typename P>
+__device__ inline float chan_map_apply(const Op &op, const P &p, float x, float y, float z, uint32_t s, float old) {
+  if constexpr (NIN >= 3) {
+    return ACC ? op.accum3(p, x, y, z, s, old) : op.value3(p, x, y, z, s);
+  } else {
+    return ACC ? op.accum(p, x, y, s, old) : op.value(p, x, y, s);
+  }
+}
+
 template <typename V, int NIN, bool ACC, int UNROLL, typename Op>
 __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
                                                           FastDiv div_c, Op op, const float *a_,
-                                                          const float *b_, float *out_, int nt) {
+                                                          const float *b_, const float *c_, float *out_, int nt) {
   constexpr int L = VecLanes<V>::n;
   const V *a = reinterpret_cast<const V *>(a_);
   const V *b = reinterpret_cast<const V *>(b_);
+  const V *c3 = reinterpret_cast<const V *>(c_);
   V *out = reinterpret_cast<V *>(out_);
   const uint32_t S = div_s.d, C = div_c.d;
   constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
   const uint32_t stride = gridDim.x * kTile;
   for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
-    V va[UNROLL], vb[UNROLL], vo[UNROLL];
+    V va[UNROLL], vb[UNROLL], vc[UNROLL], vo[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
         if (NIN >= 1) va[u] = load_stream(&a[g], nt);
         if (NIN >= 2) vb[u] = load_stream(&b[g], nt);
+        if (NIN >= 3) vc[u] = load_stream(&c3[g], nt);
         if (ACC) vo[u] = load_stream(&out[g], nt);
       }
     }
@@ -73,7 +85,8 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
         for (int k = 0; k < L; ++k) {
           const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
           const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
-          const float v = ACC ? op.accum(p, x, y, s, lane_get<V>(vo[u], k)) : op.value(p, x, y, s);
+          const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
+          const float v = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? lane_get<V>(vo[u], k) : 0.0f);
           lane_set<V>(r, k, v);
           if (k + 1 < L) {
             if (++s == S) {
@@ -95,36 +108,38 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
     const typename Op::Param p = op.load(c);
     const float x = (NIN >= 1) ? a_[i] : 0.0f;
     const float y = (NIN >= 2) ? b_[i] : 0.0f;
-    out_[i] = ACC ? op.accum(p, x, y, s, out_[i]) : op.value(p, x, y, s);
+    const float z = (NIN >= 3) ? c_[i] : 0.0f;
+    out_[i] = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? out_[i] : 0.0f);
   }
 }
 
 // a, b may be null when NIN says they are unused.
 template <int NIN, bool ACC, typename Op>
 void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
-                     const float *b, float *out, CUstream_st *stream) {
+                     const float *b, float *out, CUstream_st *stream, const float *c = nullptr) {
   const uint32_t len = checked_len(S, C, N, symbol);
   if (len == 0) return;
   const Tuning &t = tuning();
   hipStream_t s = as_stream(stream);
   const FastDiv div_s(S), div_c(C);
-  const bool vec = aligned16(out) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
+  const bool vec = aligned16(out) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b)) &&
+                   (NIN < 3 || aligned16(c));
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
     if (t.flat_unroll >= 4) {
       chan_map_kernel<f32x4, NIN, ACC, 4, Op>
-          <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+          <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
     } else if (t.flat_unroll >= 2) {
       chan_map_kernel<f32x4, NIN, ACC, 2, Op>
-          <<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+          <<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
     } else {
       chan_map_kernel<f32x4, NIN, ACC, 1, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, out, nt);
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
     }
   } else {
     chan_map_kernel<float, NIN, ACC, 4, Op>
-        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, out, 0);
+        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out, 0);
   }
   note_launch(symbol);
 }

@@ -53,15 +53,27 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
 #if defined(__HIPCC__)
 
 // Op concept:
-//   static constexpr int NIN  (1 or 2 element inputs), NACC (1 or 2 sums);
+//   static constexpr int NIN  (1 to 3 element inputs), NACC (1 to 3 sums);
 //   struct Param;  __device__ Param load(uint32_t c) const;
-//   __device__ void term(const Param&, float a, float b, double &s0, double &s1) const;
-//   __device__ void finalize(uint32_t c, double s0, double s1) const;   // writes the output(s)
+//   __device__ void term(const Param&, float a, float b, double &s0, double &s1, double &s2) const;
+//     (NIN == 3: term3(const Param&, float a, float b, float c, double &s0, double &s1, double &s2))
+//   __device__ void finalize(uint32_t c, double s0, double s1, double s2) const;   // writes the output(s)
+
+template <typename Op, typename P>
+__device__ inline void chan_reduce_term(const Op &op, const P &prm, float a, float b, float c, double &s0,
+                                        double &s1, double &s2) {
+  if constexpr (Op::NIN >= 3) {
+    op.term3(prm, a, b, c, s0, s1, s2);
+  } else {
+    op.term(prm, a, b, s0, s1, s2);
+  }
+}
 
 template <typename Op, typename V>
 __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
+                                                                   const float *__restrict__ c3,
                                                                    double *__restrict__ part, int policy) {
   constexpr int W = VecLanes<V>::n;
   constexpr int U = 4;
@@ -78,22 +90,24 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
   const uint32_t n1 = min(pl.N, n0 + pl.NB);
   const typename Op::Param prm = op.load(c);
 
-  double acc0[U], acc1[U];
+  double acc0[U], acc1[U], acc2[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) acc0[u] = acc1[u] = 0.0;
+  for (int u = 0; u < U; ++u) acc0[u] = acc1[u] = acc2[u] = 0.0;
 
   for (uint32_t n = n0; n < n1; ++n) {
     const size_t row = (size_t(n) * pl.C + c) * pl.S + s0;
     const V *pa = reinterpret_cast<const V *>(a + row);
     const V *pb = reinterpret_cast<const V *>(b + row);
+    const V *pc = reinterpret_cast<const V *>(c3 + row);
     for (uint32_t jb = 0; jb < LG; jb += uint32_t(U) * kBlock) {
-      V va[U], vb[U];
+      V va[U], vb[U], vc[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
         if (j < LG) {
           va[u] = load_stream(&pa[j], policy);
           if (Op::NIN >= 2) vb[u] = load_stream(&pb[j], policy);
+          if (Op::NIN >= 3) vc[u] = load_stream(&pc[j], policy);
         }
       }
 #pragma unroll
@@ -102,8 +116,8 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
         if (j < LG) {
 #pragma unroll
           for (int k = 0; k < W; ++k) {
-            op.term(prm, lane_get<V>(va[u], k), (Op::NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f, acc0[u],
-                    acc1[u]);
+            chan_reduce_term(op, prm, lane_get<V>(va[u], k), (Op::NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f,
+                             (Op::NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f, acc0[u], acc1[u], acc2[u]);
           }
         }
       }
@@ -112,15 +126,19 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
 
   double t0 = (acc0[0] + acc0[1]) + (acc0[2] + acc0[3]);
   double t1 = (acc1[0] + acc1[1]) + (acc1[2] + acc1[3]);
+  double t2 = (acc2[0] + acc2[1]) + (acc2[2] + acc2[3]);
   t0 = block_sum(t0, lds);
   if (Op::NACC >= 2) t1 = block_sum(t1, lds);
+  if (Op::NACC >= 3) t2 = block_sum(t2, lds);
   if (threadIdx.x == 0) {
     if (pl.ppc == 1) {
-      op.finalize(c, t0, t1);
+      op.finalize(c, t0, t1, t2);
     } else {
+      const size_t plane = size_t(pl.C) * pl.ppc;
       const size_t slot = size_t(c) * pl.ppc + (nt * pl.n_stiles + st);
       part[slot] = t0;
-      if (Op::NACC >= 2) part[size_t(pl.C) * pl.ppc + slot] = t1;
+      if (Op::NACC >= 2) part[plane + slot] = t1;
+      if (Op::NACC >= 3) part[2 * plane + slot] = t2;
     }
   }
 }
@@ -129,6 +147,7 @@ template <typename Op, typename V>
 __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl, FastDiv div_s, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
+                                                                   const float *__restrict__ c3,
                                                                    double *__restrict__ part, int policy) {
   constexpr int W = VecLanes<V>::n;
   constexpr int G = 16 / W;                       // position groups owned by a thread
@@ -145,7 +164,7 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
   const size_t CS = size_t(pl.C) * pl.S;
   const size_t p0 = size_t(c0) * pl.S;
 
-  double acc0[G][W], acc1[G][W];
+  double acc0[G][W], acc1[G][W], acc2[G][W];
   typename Op::Param prm[G][W];
   bool valid[G];
 #pragma unroll
@@ -154,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
     valid[i] = j < LG;
 #pragma unroll
     for (int k = 0; k < W; ++k) {
-      acc0[i][k] = acc1[i][k] = 0.0;
+      acc0[i][k] = acc1[i][k] = acc2[i][k] = 0.0;
       // positions past the tile read channel c0's parameters and are never used
       const uint32_t pos = valid[i] ? j * uint32_t(W) + uint32_t(k) : 0u;
       prm[i][k] = op.load(c0 + div_s.div(pos));
@@ -162,17 +181,19 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
   }
 
   for (uint32_t n = n0; n < n1; n += uint32_t(STAGES)) {
-    V va[STAGES][G], vb[STAGES][G];
+    V va[STAGES][G], vb[STAGES][G], vc[STAGES][G];
 #pragma unroll
     for (int sg = 0; sg < STAGES; ++sg) {
       if (n + uint32_t(sg) < n1) {
         const V *pa = reinterpret_cast<const V *>(a + (size_t(n + sg) * CS + p0));
         const V *pb = reinterpret_cast<const V *>(b + (size_t(n + sg) * CS + p0));
+        const V *pc = reinterpret_cast<const V *>(c3 + (size_t(n + sg) * CS + p0));
 #pragma unroll
         for (int i = 0; i < G; ++i) {
           if (valid[i]) {
             va[sg][i] = load_stream(&pa[threadIdx.x + uint32_t(i) * kBlock], policy);
             if (Op::NIN >= 2) vb[sg][i] = load_stream(&pb[threadIdx.x + uint32_t(i) * kBlock], policy);
+            if (Op::NIN >= 3) vc[sg][i] = load_stream(&pc[threadIdx.x + uint32_t(i) * kBlock], policy);
           }
         }
       }
@@ -185,8 +206,10 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
           if (valid[i]) {
 #pragma unroll
             for (int k = 0; k < W; ++k) {
-              op.term(prm[i][k], lane_get<V>(va[sg][i], k),
-                      (Op::NIN >= 2) ? lane_get<V>(vb[sg][i], k) : 0.0f, acc0[i][k], acc1[i][k]);
+              chan_reduce_term(op, prm[i][k], lane_get<V>(va[sg][i], k),
+                               (Op::NIN >= 2) ? lane_get<V>(vb[sg][i], k) : 0.0f,
+                               (Op::NIN >= 3) ? lane_get<V>(vc[sg][i], k) : 0.0f, acc0[i][k], acc1[i][k],
+                               acc2[i][k]);
             }
           }
         }
@@ -199,7 +222,7 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
   while (tpc > 1 && tpc * cb > uint32_t(kBlock)) tpc >>= 1;
   const uint32_t cl = threadIdx.x / tpc;
   const uint32_t jj = threadIdx.x % tpc;
-  double res[2] = {0.0, 0.0};
+  double res[3] = {0.0, 0.0, 0.0};
 #pragma unroll
   for (int q = 0; q < Op::NACC; ++q) {
     __syncthreads();
@@ -208,7 +231,8 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
       if (valid[i]) {
 #pragma unroll
         for (int k = 0; k < W; ++k) {
-          lds[(threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W) + uint32_t(k)] = q ? acc1[i][k] : acc0[i][k];
+          lds[(threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W) + uint32_t(k)] =
+              q == 0 ? acc0[i][k] : (q == 1 ? acc1[i][k] : acc2[i][k]);
         }
       }
     }
@@ -223,11 +247,13 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
   if (cl < cb && jj == 0) {
     const uint32_t c = c0 + cl;
     if (pl.ppc == 1) {
-      op.finalize(c, res[0], res[1]);
+      op.finalize(c, res[0], res[1], res[2]);
     } else {
+      const size_t plane = size_t(pl.C) * pl.ppc;
       const size_t slot = size_t(c) * pl.ppc + nt;
       part[slot] = res[0];
-      if (Op::NACC >= 2) part[size_t(pl.C) * pl.ppc + slot] = res[1];
+      if (Op::NACC >= 2) part[plane + slot] = res[1];
+      if (Op::NACC >= 3) part[2 * plane + slot] = res[2];
     }
   }
 }
@@ -240,27 +266,31 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_fold_kernel(uint32_t C, ui
   const uint32_t c = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   if (c >= C) return;  // uniform per wave
-  double s0 = 0.0, s1 = 0.0;
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0;
   const double *p0 = part + size_t(c) * ppc;
   const double *p1 = p0 + size_t(C) * ppc;
+  const double *p2 = p1 + size_t(C) * ppc;
   for (uint32_t j = lane; j < ppc; j += kWave) {
     s0 += p0[j];
     if (Op::NACC >= 2) s1 += p1[j];
+    if (Op::NACC >= 3) s2 += p2[j];
   }
   s0 = wave_sum(s0);
   if (Op::NACC >= 2) s1 = wave_sum(s1);
-  if (lane == 0) op.finalize(c, s0, s1);
+  if (Op::NACC >= 3) s2 = wave_sum(s2);
+  if (lane == 0) op.finalize(c, s0, s1, s2);
 }
 
 template <typename Op>
 void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
-                        const float *b, CUstream_st *stream) {
+                        const float *b, CUstream_st *stream, const float *c = nullptr) {
   const uint32_t len = checked_len(S, C, N, symbol);
   if (len == 0) return;
   hipStream_t s = as_stream(stream);
-  const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b));
+  const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b)) && (Op::NIN < 3 || aligned16(c));
   const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
   if (Op::NIN < 2) b = a;
+  if (Op::NIN < 3) c = a;
   const int nt = stream_policy(size_t(len) * sizeof(float), tuning().reduce_nontemporal);
 
   ScratchLease lease{nullptr, std::unique_lock<std::mutex>()};
@@ -272,15 +302,15 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
   if (pl.whole) {
     const FastDiv div_s(S);
     if (pl.vec) {
-      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part, nt);
+      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part, nt);
     } else {
-      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, part, nt);
+      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part, nt);
     }
   } else {
     if (pl.vec) {
-      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part, nt);
+      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part, nt);
     } else {
-      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, part, nt);
+      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part, nt);
     }
   }
   note_launch(symbol);

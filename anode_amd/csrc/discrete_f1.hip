@@ -46,11 +46,11 @@ struct F1Reduce {
   float *y;
   double eps;
   __device__ Param load(uint32_t) const { return Param{}; }
-  __device__ void term(const Param &, float a, float b, double &s0, double &s1) const {
+  __device__ void term(const Param &, float a, float b, double &s0, double &s1, double &) const {
     s0 = fma(double(a), double(b), s0);
     s1 += double(a) + double(b);
   }
-  __device__ void finalize(uint32_t c, double s0, double s1) const { y[c] = float(-(2.0 * s0 + eps) / (s1 + eps)); }
+  __device__ void finalize(uint32_t c, double s0, double s1, double) const { y[c] = float(-(2.0 * s0 + eps) / (s1 + eps)); }
 };
 
 // f1.cu:89-115 as a channel-indexed map over [S = dim0, C = K*N, 1]:

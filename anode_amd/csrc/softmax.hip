@@ -240,11 +240,16 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
 
 // C <= CMAX: the pixel's classes stay in registers, x is read once.  The sum
 // of exponentials is formed class by class in index order; the normalisation
-// multiplies by one correctly rounded reciprocal per pixel.
-template <int CMAX, typename V>
+// multiplies by one correctly rounded reciprocal per pixel.  With NLL the
+// label gather is fused: nll = -log(the stored probability of the label), NaN
+// when the label is out of range, exactly what the separate gather returns.
+template <int CMAX, typename V, bool NLL>
 __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
-                                                                float *__restrict__ y) {
+                                                                float *__restrict__ y,
+                                                                const uint32_t *__restrict__ cat,
+                                                                float *__restrict__ nll) {
   constexpr int W = PixVec<V>::W;
+  typedef typename PixVec<V>::U U;
   const uint32_t stride = gridDim.x * kBlock;
   for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
@@ -268,9 +273,29 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
       }
     }
     const V inv = vrcp(s);
+    U lab;
+    V picked = PixVec<V>::splat(0.0f);
+    if (NLL) lab = *reinterpret_cast<const U *>(cat + (size_t(p) + size_t(pg.P) * n));
 #pragma unroll
     for (int k = 0; k < CMAX; ++k) {
-      if (uint32_t(k) < pg.C) *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = v[k] * inv;
+      if (uint32_t(k) < pg.C) {
+        const V pr = v[k] * inv;
+        *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = pr;
+        if (NLL) {
+#pragma unroll
+          for (int w = 0; w < W; ++w) {
+            if (lane_get_u(lab, w) == uint32_t(k)) lane_set<V>(picked, w, lane_get<V>(pr, w));
+          }
+        }
+      }
+    }
+    if (NLL) {
+      V out;
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(lane_get<V>(picked, w)) : __builtin_nanf(""));
+      }
+      *reinterpret_cast<V *>(nll + (size_t(p) + size_t(pg.P) * n)) = out;
     }
   }
 }
@@ -360,22 +385,32 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W) {
 // one pixel group per thread: the hardware dispatcher walks the array in order
 uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
-template <typename V>
-void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, hipStream_t s) {
+// C <= 32 only
+template <typename V, bool NLL>
+void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
+                           float *nll, hipStream_t s) {
   const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
   const uint32_t blocks = pixel_blocks(pg.total_groups);
   if (C <= 4) {
-    softmax_nd_reg_kernel<4, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    softmax_nd_reg_kernel<4, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 8) {
-    softmax_nd_reg_kernel<8, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    softmax_nd_reg_kernel<8, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 16) {
-    softmax_nd_reg_kernel<16, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    softmax_nd_reg_kernel<16, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 24) {
-    softmax_nd_reg_kernel<24, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
-  } else if (C <= 32) {
-    softmax_nd_reg_kernel<32, V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    softmax_nd_reg_kernel<24, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else {
-    softmax_nd_stream_kernel<V><<<blocks, kBlock, 0, s>>>(pg, x, y);
+    softmax_nd_reg_kernel<32, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+  }
+}
+
+template <typename V>
+void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, hipStream_t s) {
+  if (C <= 32) {
+    launch_softmax_nd_reg<V, false>(P, C, N, x, y, nullptr, nullptr, s);
+  } else {
+    const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
+    softmax_nd_stream_kernel<V><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, x, y);
   }
 }
 
@@ -395,9 +430,9 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
     const uint32_t blocks = pixel_blocks(pg.total_groups);
     if (C <= 64) {
-      softmax_nd_reg_kernel<64, float><<<blocks, kBlock, 0, s>>>(pg, x, y);
+      softmax_nd_reg_kernel<64, float, false><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     } else {
-      softmax_nd_reg_kernel<128, float><<<blocks, kBlock, 0, s>>>(pg, x, y);
+      softmax_nd_reg_kernel<128, float, false><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     }
   } else if (vec) {
     launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
@@ -502,4 +537,28 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_
                                                                          const KernelConfig *,
                                                                          CUstream_st *stream) {
   launch_softmax_nd_cat_nll_bwd<true>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream);
+}
+
+// Additive (no counterpart in the reference): softmax_nd and softmax_nd_cat_nll in one pass over x.
+// Writes the same probabilities and the same nll values as the two separate entry points.
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
+                                                                const float *x, const uint32_t *cat_data,
+                                                                float *softmax, float *nll, const KernelConfig *cfg,
+                                                                CUstream_st *stream) {
+  const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
+  if (len == 0) return;
+  if (prefix_dim > 1 && dim0 <= 32) {
+    hipStream_t s = as_stream(stream);
+    const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) && aligned16(nll);
+    if (vec) {
+      launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
+    } else {
+      launch_softmax_nd_reg<float, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
+    }
+    note_launch(__func__);
+  } else {
+    // shapes outside the register-resident kernel: the two passes, back to back
+    anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
+    anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
+  }
 }

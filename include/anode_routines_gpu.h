@@ -178,6 +178,59 @@ void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_t prefix_dim,
 /* Part 2: additive entry points (no counterpart in the reference)       */
 /* ===================================================================== */
 
+/* ---- declared but never implemented by the reference (commented out in lib.h) ---- */
+
+/* lib.h:197-204 (commented out).  y[i,b] = lx[b] * rx[i,b] over [inner_dim, bcast_dim] */
+void anode_gpu_bcast_flat_mult_I1b_I2ab_Oab_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, const float *lx, const float *rx, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:205-213 (commented out).  y[i,b] = fma(lx[b], rx[i,b], shift[b]) */
+void anode_gpu_bcast_flat_mult_add_I1b_I2ab_Oab_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, const float *lx, const float *rx, const float *shift, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:214-222 (commented out).  y[i,b,o] = lx[b] * rx[i,b,o] over [inner_dim, bcast_dim, outer_dim] */
+void anode_gpu_bcast_flat_mult_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, uint32_t outer_dim, const float *lx, const float *rx, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:223-232 (commented out).  y[i,b,o] = fma(lx[b], rx[i,b,o], shift[b]): the per-channel affine (gamma, beta) */
+void anode_gpu_bcast_flat_mult_add_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, uint32_t outer_dim, const float *lx, const float *rx, const float *shift, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:235-241 (commented out).  y = lx * rx */
+void anode_gpu_flat_mult_f32(uint32_t len, const float *lx, const float *rx, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:242-249 (commented out).  y = fma(lx, rx, shift) */
+void anode_gpu_flat_mult_add_f32(uint32_t len, const float *lx, const float *rx, const float *shift, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:408-414 (commented out).  y[b] = sum_a x[a,b] */
+void anode_gpu_sum_Iab_Ob_packed_deterministic_f32(uint32_t reduce_dim, uint32_t outer_dim, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:415-422 (commented out).  y[b] = sum_{a,c} x[a,b,c] */
+void anode_gpu_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, uint32_t mid_dim, uint32_t reduce_outer_dim, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* lib.h:423-430 (commented out).  y[b] = sum_{a,c} x[a,b,c]^2 */
+void anode_gpu_square_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, uint32_t mid_dim, uint32_t reduce_outer_dim, const float *x, float *y, ANODE_LAUNCH_TAIL);
+
+/* ---- no counterpart in the reference ---- */
+
+/* Inverse of dequantize: scale = (hi-lo)/255; y = clamp(rint((x-lo)/scale), 0, 255), round half to even, NaN -> 0. */
+void anode_gpu_quantize_u8_packed_f32(uint32_t len, float lo, float hi, const float *x, uint8_t *y, ANODE_LAUNCH_TAIL);
+/* u8 image normalisation in one pass: y[i,b,o] = fma(scale[b], float(x[i,b,o]), shift[b]). */
+void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, uint32_t outer_dim, const float *scale, const float *shift, const uint8_t *x, float *y, ANODE_LAUNCH_TAIL);
+/* batch_mean and batch_var in one pass over x: mean[c], var[c] = biased variance + epsilon (composes with batch_norm). */
+void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, float *mean, float *var, ANODE_LAUNCH_TAIL);
+/* batch_norm followed by positive_clip in one pass: t = (x-mean[c])*rsqrt(var[c]); y = t * float(t>0). */
+void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, const float *mean, const float *var, float *y, ANODE_LAUNCH_TAIL);
+/* batch_norm followed by the per-channel affine in one pass: y = fma((x-mean[c])*rsqrt(var[c]), gamma[c], beta[c]). */
+void anode_gpu_batch_norm_affine_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, const float *mean, const float *var, const float *gamma, const float *beta, float *y, ANODE_LAUNCH_TAIL);
+/* The three backward reductions in one pass over (dy, x): dvar = batch_norm_bwd_var; dmean = batch_norm_bwd_mean +
+ * batch_var_bwd_mean(dvar).  mask may be NULL; otherwise dy is first multiplied by float(mask>0) (ReLU backward). */
+void anode_gpu_batch_norm_bwd_reduce_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, const float *mask, float *dmean, float *dvar, ANODE_LAUNCH_TAIL);
+/* The three backward maps in one pass: dx = batch_norm_bwd + batch_var_bwd(dvar) + batch_mean_bwd(dmean), the terms
+ * formed and added exactly as the three separate launches do.  mask as above. */
+void anode_gpu_batch_norm_bwd_apply_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, const float *dmean, const float *dvar, const float *mask, float *dx, ANODE_LAUNCH_TAIL);
+/* dx += ... */
+void anode_gpu_batch_norm_bwd_apply_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, const float *dmean, const float *dvar, const float *mask, float *dx, ANODE_LAUNCH_TAIL);
+/* softmax_nd and softmax_nd_cat_nll in one pass over x; writes the same softmax and nll as the two entry points. */
+void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, float *softmax, float *nll, ANODE_LAUNCH_TAIL);
+/* Running statistics: y <- fma(rate, x - y, y) (the semantics of anode's online_average, tests/test_gpu.rs:561-593). */
+void anode_gpu_online_average_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* Device form of the host rule src/utils/mod.rs:31-41 per row of a [dim0 (fastest), dim1] array: first index of the
+ * strict maximum, NaN never selected, 0 when nothing exceeds -inf. */
+void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, const float *x, uint32_t *index, ANODE_LAUNCH_TAIL);
+
+/* The host-side rule itself (src/utils/mod.rs:31-41), for logits already on the host: first index of the strict
+ * maximum starting from (-inf, 0); NaN never selected.  xs is a HOST pointer. */
+size_t anode_host_arg_max_f32(const float *xs, size_t len);
+
 /* Library introspection.  No reference counterpart. */
 /* 0 when no launch made by this library has failed since the last call; otherwise the hipError_t
  * of the most recent failed launch.  Reading clears it. */

@@ -877,6 +877,29 @@ ORACLE_API void oracle_batch_mean_var_f64(uint32_t d0, uint32_t d1, uint32_t d2,
                   var[c] = accumulator / n + (double)eps);
 }
 
+/* the commented-out declarations lib.h:408-430: y[b] = sum_{a,c} x[a,b,c] (or of x^2), in double */
+ORACLE_API void oracle_channel_sum_f64(uint32_t d0, uint32_t d1, uint32_t d2, int square, const float *x,
+                                       double *y) {
+  CHANNEL_SUM_F64(d0, d1, d2, (void)0, square ? (double)x[idx] * (double)x[idx] : (double)x[idx],
+                  y[c] = accumulator);
+}
+
+/* batch_norm followed by the per-channel affine: y = fma((x-m)*rs, gamma[c], beta[c]) */
+ORACLE_API void oracle_batch_norm_affine_f32ref(uint32_t d0, uint32_t d1, uint32_t d2, const float *x,
+                                                const float *mean, const float *var, const float *gamma,
+                                                const float *beta, float *y) {
+  CHANNEL_MAP(d0, d1, d2,
+              { y[idx] = fmaf((x[idx] - mean[c]) * rsqrt_f32(var[c]), gamma[c], beta[c]); });
+}
+
+ORACLE_API void oracle_batch_norm_affine_f64(uint32_t d0, uint32_t d1, uint32_t d2, const float *x,
+                                             const float *mean, const float *var, const float *gamma,
+                                             const float *beta, double *y) {
+  CHANNEL_MAP(d0, d1, d2, {
+    y[idx] = ((double)x[idx] - (double)mean[c]) / sqrt((double)var[c]) * (double)gamma[c] + (double)beta[c];
+  });
+}
+
 /* running statistics, semantics fixed by tests/test_gpu.rs:561-593:
  * y <- y + rate * (x - y) */
 ORACLE_API void oracle_online_average(uint32_t len, float rate, const float *x, float *y) {

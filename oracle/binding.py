@@ -405,3 +405,18 @@ def online_average(rate, x, y):
     out = _f32(y).ravel().copy()
     lib().oracle_online_average(u32(x.size), f32(rate), _p(x), _p(out))
     return out
+
+
+def channel_sum(d0, d1, d2, x, square=False):
+    x = _f32(x)
+    out = np.empty(d1, np.float64)
+    lib().oracle_channel_sum_f64(u32(d0), u32(d1), u32(d2), cint(int(square)), _p(x), _p(out))
+    return out
+
+
+def batch_norm_affine(d0, d1, d2, x, mean, var, gamma, beta, f64=False):
+    x, mean, var, gamma, beta = _f32(x), _f32(mean), _f32(var), _f32(gamma), _f32(beta)
+    out = np.empty(d0 * d1 * d2, np.float64 if f64 else np.float32)
+    fn = lib().oracle_batch_norm_affine_f64 if f64 else lib().oracle_batch_norm_affine_f32ref
+    fn(u32(d0), u32(d1), u32(d2), _p(x), _p(mean), _p(var), _p(gamma), _p(beta), _p(out))
+    return out

@@ -147,6 +147,24 @@ def test_reduction_entry_points_abort_on_non_power_of_two_block(name):
     assert "returned" not in r.stdout
 
 
+def test_host_arg_max_follows_the_reference_rule():
+    # src/utils/mod.rs:31-41: start from (-inf, 0); strictly greater wins; NaN never wins
+    fn = _lib.load().symbol("anode_host_arg_max_f32")
+
+    def arg_max(values):
+        a = np.asarray(values, np.float32)
+        return fn(a.ctypes.data, a.size)
+
+    assert arg_max([1, 3, 3, 2]) == 1
+    assert arg_max([-np.inf, -np.inf]) == 0
+    assert arg_max([np.nan, 1.0, np.nan, 1.0]) == 1
+    assert arg_max([np.nan, np.nan]) == 0
+    assert arg_max([]) == 0
+    assert arg_max([-1, -0.0, 0.0]) == 1
+    x = np.random.default_rng(0).standard_normal(1000).astype(np.float32)
+    assert arg_max(x) == int(np.argmax(x))
+
+
 def test_exact_division_helper_matches_integer_division():
     probe = _lib.load().cdll.anode_gpu_fastdiv_probe
     g = np.random.default_rng(0)
