@@ -322,17 +322,33 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
   }
 }
 
-// softmax.cu:278-298: per-pixel gather; one thread per pixel
+// softmax.cu:278-298: per-pixel gather.  A thread takes W consecutive pixels:
+// one 16-byte label load, W independent gathers in flight, one 16-byte store.
+template <typename V>
 __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg, const float *__restrict__ prob,
                                                                     const uint32_t *__restrict__ cat,
                                                                     float *__restrict__ nll) {
+  constexpr int W = PixVec<V>::W;
+  typedef typename PixVec<V>::U U;
   const uint32_t stride = gridDim.x * kBlock;
   for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
-    pixel_decode(pg, g, 1, p, n);
-    const uint32_t k = cat[g];
-    nll[g] = (k < pg.C) ? -logf(prob[size_t(p) + size_t(pg.P) * (size_t(k) + size_t(pg.C) * n)])
-                        : __builtin_nanf("");
+    pixel_decode(pg, g, W, p, n);
+    const size_t pix = size_t(p) + size_t(pg.P) * n;
+    const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
+    const U lab = *reinterpret_cast<const U *>(cat + pix);
+    float pr[W];
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      const uint32_t k = lane_get_u(lab, w);
+      pr[w] = (k < pg.C) ? prob[base + size_t(w) + size_t(pg.P) * k] : 0.0f;
+    }
+    V out;
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr[w]) : __builtin_nanf(""));
+    }
+    *reinterpret_cast<V *>(nll + pix) = out;
   }
 }
 
@@ -518,8 +534,15 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_packed_f32(uint32_t prefix_dim, u
                                                           float *nll, const KernelConfig *, CUstream_st *stream) {
   (void)checked_len(prefix_dim, dim0, dim1, __func__);
   if (prefix_dim == 0 || dim1 == 0) return;
-  const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 1);
-  softmax_nd_cat_nll_kernel<<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
+  if (prefix_dim % 4 == 0 && aligned16(cat_data) && aligned16(nll)) {
+    const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 4);
+    softmax_nd_cat_nll_kernel<f32x4>
+        <<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
+  } else {
+    const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 1);
+    softmax_nd_cat_nll_kernel<float>
+        <<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
+  }
   note_launch(__func__);
 }
 

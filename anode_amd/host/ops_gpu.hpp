@@ -1,0 +1,492 @@
+// Host side above the C ABI, in C++: the caller layer of anode's
+// src/ops_gpu.rs for the operators of routines_gpu, with the same operator
+// names, the same dimension mapping, the same Assign / Accumulate dispatch and
+// the same failure behaviour (the reference's `unimplemented!()` and `assert!`
+// become exceptions).  It owns no memory and launches nothing itself: every
+// apply() ends in one call of an `anode_gpu_*` entry point, exactly where the
+// Rust closure makes its `unsafe { anode_gpu_*(...) }` call.
+//
+// Arrays are the reference's packed, first-index-fastest arrays
+// (GPUDeviceOuterBatchArray{1,3,4}d: `size` = the non-batch dimensions, fastest
+// first, plus a batch size), described here by a device pointer and a Shape.
+#pragma once
+
+#define ANODE_DEFINE_KERNEL_CONFIG
+#include "../../include/anode_routines_gpu.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+namespace anode_host {
+
+// src/lib.rs:1810-1813
+enum class WriteCap { Assign, Accumulate };
+
+// the reference's `unimplemented!()`
+struct Unimplemented : std::logic_error {
+  explicit Unimplemented(const std::string &what) : std::logic_error("unimplemented: " + what) {}
+};
+
+// src/ops_gpu.rs:57-61: sizes must fit the ABI's u32
+inline uint32_t sz2uint(size_t sz) {
+  if (sz > 0xffffffffull) throw std::overflow_error("sz2uint: size does not fit in u32");
+  return uint32_t(sz);
+}
+
+// What the Rust callers take from their connection: conn.cuda_stream() and
+// conn.cuda_kernel_config() (src/ops_gpu.rs:670-679).
+struct GPUDeviceConn {
+  hipStream_t stream = nullptr;
+  KernelConfig cfg{1024, 1024};
+  const KernelConfig *cuda_kernel_config() const { return &cfg; }
+  CUstream_st *cuda_stream() const { return reinterpret_cast<CUstream_st *>(stream); }
+};
+
+// Non-batch dimensions (fastest first) and the outer batch size.
+struct Shape {
+  size_t size[4] = {1, 1, 1, 1};
+  int nd = 1;
+  size_t batch = 1;
+  size_t index_at(int i) const { return i < nd ? size[i] : batch; }  // the batch is the last axis
+  size_t flat_len_upto(int n) const {                                // product of the first n axes
+    size_t p = 1;
+    for (int i = 0; i < n; ++i) p *= size[i];
+    return p;
+  }
+  size_t flat_len() const { return flat_len_upto(nd) * batch; }
+};
+
+template <typename T>
+struct DeviceArray {
+  T *dptr = nullptr;
+  Shape shape;
+  bool packed = true;  // only packed arrays are implemented, as in the reference
+  bool is_packed() const { return packed; }
+  const T *as_dptr() const { return dptr; }
+  T *as_mut_dptr() const { return dptr; }
+};
+
+inline DeviceArray<float> array1d(float *p, size_t n) {
+  DeviceArray<float> a;
+  a.dptr = p;
+  a.shape.size[0] = n;
+  a.shape.nd = 1;
+  return a;
+}
+
+// [d0, batch]: GPUDeviceOuterBatchArray1d
+template <typename T>
+inline DeviceArray<T> obatch1d(T *p, size_t d0, size_t batch) {
+  DeviceArray<T> a;
+  a.dptr = p;
+  a.shape.size[0] = d0;
+  a.shape.nd = 1;
+  a.shape.batch = batch;
+  return a;
+}
+
+// [W, H, C, batch]: GPUDeviceOuterBatchArray3d (NCHW memory)
+template <typename T>
+inline DeviceArray<T> obatch3d(T *p, size_t w, size_t h, size_t c, size_t batch) {
+  DeviceArray<T> a;
+  a.dptr = p;
+  a.shape.size[0] = w;
+  a.shape.size[1] = h;
+  a.shape.size[2] = c;
+  a.shape.nd = 3;
+  a.shape.batch = batch;
+  return a;
+}
+
+// [X, Y, Z, C, batch]: GPUDeviceOuterBatchArray4d (NCDHW memory)
+template <typename T>
+inline DeviceArray<T> obatch4d(T *p, size_t x, size_t y, size_t z, size_t c, size_t batch) {
+  DeviceArray<T> a;
+  a.dptr = p;
+  a.shape.size[0] = x;
+  a.shape.size[1] = y;
+  a.shape.size[2] = z;
+  a.shape.size[3] = c;
+  a.shape.nd = 4;
+  a.shape.batch = batch;
+  return a;
+}
+
+namespace detail {
+template <typename... A>
+inline void require_packed(const char *op, const A &...arrays) {
+  const bool packed = (arrays.is_packed() && ...);
+  if (!packed) throw Unimplemented(std::string(op) + ": non-packed arrays");
+}
+// (dim0, dim1, dim2) = (flat_len of the spatial axes, channels, batch): src/ops_gpu.rs:3764-3766, 4911-4913
+struct Dims3 {
+  uint32_t d0, d1, d2;
+};
+inline Dims3 spatial_channel_batch(const Shape &s) {
+  const int spatial = s.nd - 1;
+  return Dims3{sz2uint(s.flat_len_upto(spatial)), sz2uint(s.size[spatial]), sz2uint(s.batch)};
+}
+}  // namespace detail
+
+// ---------------------------------------------------------------------------
+// casts (src/ops_gpu.rs:585-967)
+// ---------------------------------------------------------------------------
+
+struct UpcastOp {  // :673
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<uint8_t> &x, DeviceArray<uint32_t> &y) {
+    detail::require_packed("UpcastOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("UpcastOp: Accumulate");
+    anode_gpu_upcast_u8_packed_u32(sz2uint(x.shape.flat_len()), x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+                                   conn.cuda_stream());
+  }
+};
+
+struct DequantizeOp {  // :762, :843
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float lo, float hi, const DeviceArray<uint8_t> &x,
+                    DeviceArray<float> &y) {
+    detail::require_packed("DequantizeOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("DequantizeOp: Accumulate");
+    anode_gpu_dequantize_u8_packed_f32(sz2uint(x.shape.flat_len()), lo, hi, x.as_dptr(), y.as_mut_dptr(),
+                                       conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct OneHotOp {  // :937-940: y is [X,Y,Z, K, batch], x is [X,Y,Z, batch]
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<uint32_t> &x, DeviceArray<float> &y) {
+    detail::require_packed("OneHotOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("OneHotOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(y.shape);
+    anode_gpu_discrete_one_hot_3d1_packed_f32(d.d0, d.d1, d.d2, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+                                              conn.cuda_stream());
+  }
+};
+
+// ---------------------------------------------------------------------------
+// batch norm pieces (src/ops_gpu.rs:3672-5860).  The 2-D and 3-D operators of
+// the reference differ only in the rank of x; one implementation serves both.
+// ---------------------------------------------------------------------------
+
+struct BatchMeanOp {  // BatchMean2dOp :3763, BatchMean3dOp :4910
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &mean) {
+    detail::require_packed("BatchMeanOp", x, mean);
+    if (cap != WriteCap::Assign) throw Unimplemented("BatchMeanOp: Accumulate");  // :3781
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_batch_mean_3d1_packed_f32(d.d0, d.d1, d.d2, x.as_dptr(), mean.as_mut_dptr(), conn.cuda_kernel_config(),
+                                        conn.cuda_stream());
+  }
+};
+
+struct BatchMeanBwdOp {  // :3865/:3880, :5012/:5027; the shape comes from x (the adjoint has x's shape)
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dmean, DeviceArray<float> &dx) {
+    detail::require_packed("BatchMeanBwdOp", dmean, dx);
+    const detail::Dims3 d = detail::spatial_channel_batch(dx.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_mean_bwd_3d1_packed_f32
+                                      : anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dmean.as_dptr(), dx.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct BatchVarianceOp {  // :3970, :5117
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float epsilon, const DeviceArray<float> &x,
+                    const DeviceArray<float> &mean, DeviceArray<float> &var) {
+    detail::require_packed("BatchVarianceOp", x, mean, var);
+    if (cap != WriteCap::Assign) throw Unimplemented("BatchVarianceOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_batch_var_3d1_packed_f32(d.d0, d.d1, d.d2, epsilon, x.as_dptr(), mean.as_dptr(), var.as_mut_dptr(),
+                                       conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct BatchVarianceBwdOp {  // :4079/:4097, :5226/:5244
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dvar, const DeviceArray<float> &x,
+                    const DeviceArray<float> &mean, DeviceArray<float> &dx) {
+    detail::require_packed("BatchVarianceBwdOp", dvar, x, mean, dx);
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_var_bwd_3d1_packed_f32
+                                      : anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dvar.as_dptr(), x.as_dptr(), mean.as_dptr(), dx.as_mut_dptr(), conn.cuda_kernel_config(),
+       conn.cuda_stream());
+  }
+};
+
+struct BatchVarianceBwdMeanOp {  // :4196/:4214, :5343/:5361
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dvar, const DeviceArray<float> &x,
+                    const DeviceArray<float> &mean, DeviceArray<float> &dmean) {
+    detail::require_packed("BatchVarianceBwdMeanOp", dvar, x, mean, dmean);
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_var_bwd_mean_3d1_packed_f32
+                                      : anode_gpu_batch_var_bwd_mean_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dvar.as_dptr(), x.as_dptr(), mean.as_dptr(), dmean.as_mut_dptr(), conn.cuda_kernel_config(),
+       conn.cuda_stream());
+  }
+};
+
+struct BatchNormalizeOp {  // :4315, :5462
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, const DeviceArray<float> &mean,
+                    const DeviceArray<float> &var, DeviceArray<float> &y) {
+    detail::require_packed("BatchNormalizeOp", x, mean, var, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("BatchNormalizeOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_batch_norm_3d1_packed_f32(d.d0, d.d1, d.d2, x.as_dptr(), mean.as_dptr(), var.as_dptr(), y.as_mut_dptr(),
+                                        conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct BatchNormalizeBwdOp {  // :4426/:4442, :5573/:5589
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &var,
+                    DeviceArray<float> &dx) {
+    detail::require_packed("BatchNormalizeBwdOp", dy, var, dx);
+    const detail::Dims3 d = detail::spatial_channel_batch(dy.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_norm_bwd_3d1_packed_f32
+                                      : anode_gpu_batch_norm_bwd_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dy.as_dptr(), var.as_dptr(), dx.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct BatchNormalizeBwdMeanOp {  // :4536/:4552, :5683/:5699
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &var,
+                    DeviceArray<float> &dmean) {
+    detail::require_packed("BatchNormalizeBwdMeanOp", dy, var, dmean);
+    const detail::Dims3 d = detail::spatial_channel_batch(dy.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_norm_bwd_mean_3d1_packed_f32
+                                      : anode_gpu_batch_norm_bwd_mean_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dy.as_dptr(), var.as_dptr(), dmean.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct BatchNormalizeBwdVarianceOp {  // :4683/:4703, :5806/:5826; build_device_f32_op_v2 :4794/:4808
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &x,
+                    const DeviceArray<float> &mean, const DeviceArray<float> &var, DeviceArray<float> &dvar) {
+    detail::require_packed("BatchNormalizeBwdVarianceOp", dy, x, mean, var, dvar);
+    const detail::Dims3 d = detail::spatial_channel_batch(dy.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_norm_bwd_var_3d1_packed_f32
+                                      : anode_gpu_batch_norm_bwd_var_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dy.as_dptr(), x.as_dptr(), mean.as_dptr(), var.as_dptr(), dvar.as_mut_dptr(),
+       conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+  static void apply_v2(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &y,
+                       const DeviceArray<float> &var, DeviceArray<float> &dvar) {
+    detail::require_packed("BatchNormalizeBwdVarianceOp(v2)", dy, y, var, dvar);
+    const detail::Dims3 d = detail::spatial_channel_batch(dy.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_batch_norm_bwd_var_v2_3d1_packed_f32
+                                      : anode_gpu_batch_norm_bwd_var_v2_3d1_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dy.as_dptr(), y.as_dptr(), var.as_dptr(), dvar.as_mut_dptr(), conn.cuda_kernel_config(),
+       conn.cuda_stream());
+  }
+};
+
+// ---------------------------------------------------------------------------
+// softmax and categorical NLL (src/ops_gpu.rs:6079-6990)
+// ---------------------------------------------------------------------------
+
+struct SoftmaxOp {  // :6153-6179: x is [K, batch]; the entry point is chosen by K <= cfg.block_sz
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("SoftmaxOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("SoftmaxOp: Accumulate");  // :6181
+    const uint32_t k = sz2uint(x.shape.index_at(0)), n = sz2uint(x.shape.index_at(1));
+    auto fn = x.shape.index_at(0) <= conn.cfg.block_sz ? anode_gpu_softmax_packed_block_f32
+                                                       : anode_gpu_softmax_packed_deterministic_f32;
+    fn(k, n, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct SoftmaxCategoricalNLLOp {  // :6275
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &softmax,
+                    const DeviceArray<uint32_t> &category_data, DeviceArray<float> &nll) {
+    detail::require_packed("SoftmaxCategoricalNLLOp", softmax, category_data, nll);
+    if (cap != WriteCap::Assign) throw Unimplemented("SoftmaxCategoricalNLLOp: Accumulate");
+    anode_gpu_softmax_cat_nll_packed_f32(sz2uint(softmax.shape.index_at(0)), sz2uint(softmax.shape.index_at(1)),
+                                         softmax.as_dptr(), category_data.as_dptr(), nll.as_mut_dptr(),
+                                         conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct SoftmaxCategoricalNLLBwdOp {  // :6379/:6396
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &softmax,
+                    const DeviceArray<uint32_t> &category_data, DeviceArray<float> &dx) {
+    detail::require_packed("SoftmaxCategoricalNLLBwdOp", dy, softmax, category_data, dx);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_softmax_cat_nll_bwd_packed_f32
+                                      : anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32;
+    fn(sz2uint(softmax.shape.index_at(0)), sz2uint(softmax.shape.index_at(1)), dy.as_dptr(), softmax.as_dptr(),
+       category_data.as_dptr(), dx.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct Softmax3dOp {  // :6492-6495: x is [X,Y,Z, C, batch] -> (prefix, C, batch)
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("Softmax3dOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("Softmax3dOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_softmax_nd_packed_f32(d.d0, d.d1, d.d2, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+                                    conn.cuda_stream());
+  }
+};
+
+struct Softmax3dCategoricalNLLOp {  // :6610, :6715
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &softmax,
+                    const DeviceArray<uint32_t> &category_data, DeviceArray<float> &nll) {
+    detail::require_packed("Softmax3dCategoricalNLLOp", softmax, category_data, nll);
+    if (cap != WriteCap::Assign) throw Unimplemented("Softmax3dCategoricalNLLOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(softmax.shape);
+    anode_gpu_softmax_nd_cat_nll_packed_f32(d.d0, d.d1, d.d2, softmax.as_dptr(), category_data.as_dptr(), nll.as_mut_dptr(),
+                                            conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct Softmax3dCategoricalNLLBwdOp {  // :6823/:6841, :6942/:6960
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &softmax,
+                    const DeviceArray<uint32_t> &category_data, DeviceArray<float> &dx) {
+    detail::require_packed("Softmax3dCategoricalNLLBwdOp", dy, softmax, category_data, dx);
+    const detail::Dims3 d = detail::spatial_channel_batch(softmax.shape);
+    auto fn = cap == WriteCap::Assign ? anode_gpu_softmax_nd_cat_nll_bwd_packed_f32
+                                      : anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32;
+    fn(d.d0, d.d1, d.d2, dy.as_dptr(), softmax.as_dptr(), category_data.as_dptr(), dx.as_mut_dptr(),
+       conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+// ---------------------------------------------------------------------------
+// smooth F1 (src/ops_gpu.rs:6991-7203)
+// ---------------------------------------------------------------------------
+
+struct NegativeF1Loss3dOp {  // :7060: x, target are [X,Y,Z, K, batch]; y is [K, batch]
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float epsilon, const DeviceArray<float> &x,
+                    const DeviceArray<float> &target, DeviceArray<float> &y) {
+    detail::require_packed("NegativeF1Loss3dOp", x, target, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("NegativeF1Loss3dOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_smooth_negative_f1_loss_3d1_packed_f32(d.d0, d.d1, d.d2, epsilon, x.as_dptr(), target.as_dptr(),
+                                                     y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct NegativeF1Loss3dBwdOp {  // :7162
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float epsilon, const DeviceArray<float> &dy,
+                    const DeviceArray<float> &x, const DeviceArray<float> &target, DeviceArray<float> &dx) {
+    detail::require_packed("NegativeF1Loss3dBwdOp", dy, x, target, dx);
+    if (cap != WriteCap::Assign) throw Unimplemented("NegativeF1Loss3dBwdOp: Accumulate");
+    const detail::Dims3 d = detail::spatial_channel_batch(x.shape);
+    anode_gpu_smooth_negative_f1_loss_3d1_bwd_packed_f32(d.d0, d.d1, d.d2, epsilon, dy.as_dptr(), x.as_dptr(),
+                                                         target.as_dptr(), dx.as_mut_dptr(), conn.cuda_kernel_config(),
+                                                         conn.cuda_stream());
+  }
+};
+
+// ---------------------------------------------------------------------------
+// flat maps and the flat join (src/ops_gpu.rs:7779-8261, 8356-9160): the
+// ApplyGPUFlatMap / ...Bwd / ...Inplace / ...BwdInplace traits as functions.
+// ---------------------------------------------------------------------------
+
+typedef void (*FlatMapFn)(uint32_t, const float *, float *, const KernelConfig *, CUstream_st *);
+typedef void (*FlatMapBwdFn)(uint32_t, const float *, const float *, float *, const KernelConfig *, CUstream_st *);
+
+template <FlatMapFn Fn>
+struct FlatMap {
+  static void apply_gpu_flat_map(const DeviceArray<float> &x, DeviceArray<float> &y, const GPUDeviceConn &conn) {
+    detail::require_packed("apply_gpu_flat_map", x, y);
+    if (x.shape.flat_len() != y.shape.flat_len()) throw std::invalid_argument("apply_gpu_flat_map: size mismatch");
+    Fn(sz2uint(x.shape.flat_len()), x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+  // :7912-7918: the output aliases the input
+  static void apply_gpu_flat_map_inplace(DeviceArray<float> &x, const GPUDeviceConn &conn) {
+    detail::require_packed("apply_gpu_flat_map_inplace", x);
+    Fn(sz2uint(x.shape.flat_len()), x.as_dptr(), x.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+template <FlatMapBwdFn Fn>
+struct FlatMapBwd {
+  static void apply_gpu_flat_map_bwd(const DeviceArray<float> &adj_y, const DeviceArray<float> &y, DeviceArray<float> &adj_x,
+                                     const GPUDeviceConn &conn) {
+    detail::require_packed("apply_gpu_flat_map_bwd", adj_y, y, adj_x);
+    Fn(sz2uint(y.shape.flat_len()), adj_y.as_dptr(), y.as_dptr(), adj_x.as_mut_dptr(), conn.cuda_kernel_config(),
+       conn.cuda_stream());
+  }
+  // :7931-7937: adj_x aliases adj_y
+  static void apply_gpu_flat_map_bwd_inplace(DeviceArray<float> &adj_y, const DeviceArray<float> &y, const GPUDeviceConn &conn) {
+    detail::require_packed("apply_gpu_flat_map_bwd_inplace", adj_y, y);
+    Fn(sz2uint(y.shape.flat_len()), adj_y.as_dptr(), y.as_dptr(), adj_y.as_mut_dptr(), conn.cuda_kernel_config(),
+       conn.cuda_stream());
+  }
+};
+
+typedef FlatMap<anode_gpu_modulus_flat_map_f32> ModulusFlatMapF;              // :7810
+typedef FlatMap<anode_gpu_square_flat_map_f32> SquareFlatMapF;                // :7830
+typedef FlatMap<anode_gpu_sqrt_flat_map_f32> SqrtFlatMap;                     // :7854
+typedef FlatMap<anode_gpu_positive_clip_flat_map_f32> PositiveClipFlatMap;    // :7873, :7912, :7947
+typedef FlatMapBwd<anode_gpu_positive_clip_flat_map_bwd_f32> PositiveClipFlatMapBwd;  // :7895, :7931
+typedef FlatMap<anode_gpu_unit_step_flat_map_f32> UnitStepFlatMapF;           // :7992
+typedef FlatMap<anode_gpu_tanh_flat_map_f32> TanhFlatMapF;                    // :8021
+typedef FlatMap<anode_gpu_rcosh2_flat_map_f32> RCosh2FlatMapF;                // :8041
+typedef FlatMap<anode_gpu_logistic_flat_map_f32> LogisticOp;                  // :9035
+typedef FlatMapBwd<anode_gpu_logistic_flat_map_bwd_f32> LogisticBwdOp;        // :9126
+
+// Map2FlatJoin<IdentityFlatMapF, UnitStepFlatMapF, ProductReduce>  :8181
+struct Map2FlatJoinIdentityUnitStepProduct {
+  static void apply_gpu_flat_join(const DeviceArray<float> &x1, const DeviceArray<float> &x2, DeviceArray<float> &y,
+                                  const GPUDeviceConn &conn) {
+    detail::require_packed("apply_gpu_flat_join", x1, x2, y);
+    anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32(sz2uint(y.shape.flat_len()), x1.as_dptr(),
+                                                                          x2.as_dptr(), y.as_mut_dptr(),
+                                                                          conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct LeakyReluOp {  // :8832
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float neg_slope, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("LeakyReluOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("LeakyReluOp: Accumulate");
+    anode_gpu_leaky_relu_flat_map_f32(sz2uint(x.shape.flat_len()), neg_slope, x.as_dptr(), y.as_mut_dptr(),
+                                      conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct LeakyReluBwdOp {  // :8924
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, float neg_slope, const DeviceArray<float> &dy,
+                    const DeviceArray<float> &y, DeviceArray<float> &dx) {
+    detail::require_packed("LeakyReluBwdOp", dy, y, dx);
+    if (cap != WriteCap::Assign) throw Unimplemented("LeakyReluBwdOp: Accumulate");
+    anode_gpu_leaky_relu_flat_map_bwd_f32(sz2uint(y.shape.flat_len()), neg_slope, dy.as_dptr(), y.as_dptr(), dx.as_mut_dptr(),
+                                          conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+// ---------------------------------------------------------------------------
+// recipes of src/ops.rs on top of the operators
+// ---------------------------------------------------------------------------
+
+// src/ops.rs:999-1014 (2-D) and :1043-1055 (3-D): mean, variance (+eps inside), normalize with the batch
+// statistics; returns nothing, fills mean / var / y.  (The running averages of the recipe are gpudevicemem's
+// online_average; anode_gpu_online_average_packed_f32 provides them here.)
+inline void batch_normalize(const GPUDeviceConn &conn, float epsilon, const DeviceArray<float> &x, DeviceArray<float> &mean,
+                            DeviceArray<float> &var, DeviceArray<float> &y) {
+  BatchMeanOp::apply(WriteCap::Assign, conn, x, mean);
+  BatchVarianceOp::apply(WriteCap::Assign, conn, epsilon, x, mean, var);
+  BatchNormalizeOp::apply(WriteCap::Assign, conn, x, mean, var, y);
+}
+
+// The adjoint graph of the recipe (src/ops_gpu.rs:4344-4352, 3997-4004, 3787-3795) in the order the sink
+// evaluates it: the first writer of each adjoint assigns, the later writers accumulate (src/lib.rs:2160-2165).
+inline void batch_normalize_adjoint(const GPUDeviceConn &conn, const DeviceArray<float> &dy, const DeviceArray<float> &x,
+                                    const DeviceArray<float> &mean, const DeviceArray<float> &var, DeviceArray<float> &dmean,
+                                    DeviceArray<float> &dvar, DeviceArray<float> &dx) {
+  BatchNormalizeBwdOp::apply(WriteCap::Assign, conn, dy, var, dx);
+  BatchNormalizeBwdMeanOp::apply(WriteCap::Assign, conn, dy, var, dmean);
+  BatchNormalizeBwdVarianceOp::apply(WriteCap::Assign, conn, dy, x, mean, var, dvar);
+  BatchVarianceBwdOp::apply(WriteCap::Accumulate, conn, dvar, x, mean, dx);
+  BatchVarianceBwdMeanOp::apply(WriteCap::Accumulate, conn, dvar, x, mean, dmean);
+  BatchMeanBwdOp::apply(WriteCap::Accumulate, conn, dmean, dx);
+}
+
+// src/ops.rs:1172-1176: p = softmax(x); nll = NLL(p, labels)
+inline void softmax_categorical_nll(const GPUDeviceConn &conn, const DeviceArray<float> &x,
+                                    const DeviceArray<uint32_t> &labels, DeviceArray<float> &softmax, DeviceArray<float> &nll) {
+  SoftmaxOp::apply(WriteCap::Assign, conn, x, softmax);
+  SoftmaxCategoricalNLLOp::apply(WriteCap::Assign, conn, softmax, labels, nll);
+}
+
+}  // namespace anode_host
