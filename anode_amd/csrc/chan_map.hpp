@@ -48,10 +48,10 @@ __device__ inline float chan_map_apply(const Op &op, const P &p, float x, float 
   }
 }
 
-template <typename V, int NIN, bool ACC, int UNROLL, typename Op>
+template <typename V, int NIN, bool ACC, int UNROLL, int NT, typename Op>
 __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
                                                           FastDiv div_c, Op op, const float *a_,
-                                                          const float *b_, const float *c_, float *out_, int nt) {
+                                                          const float *b_, const float *c_, float *out_) {
   constexpr int L = VecLanes<V>::n;
   const V *a = reinterpret_cast<const V *>(a_);
   const V *b = reinterpret_cast<const V *>(b_);
@@ -66,10 +66,10 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
     for (int u = 0; u < UNROLL; ++u) {
       const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
-        if (NIN >= 1) va[u] = load_stream(&a[g], nt);
-        if (NIN >= 2) vb[u] = load_stream(&b[g], nt);
-        if (NIN >= 3) vc[u] = load_stream(&c3[g], nt);
-        if (ACC) vo[u] = load_stream(&out[g], nt);
+        if (NIN >= 1) va[u] = load_stream<NT>(&a[g]);
+        if (NIN >= 2) vb[u] = load_stream<NT>(&b[g]);
+        if (NIN >= 3) vc[u] = load_stream<NT>(&c3[g]);
+        if (ACC) vo[u] = load_stream<NT>(&out[g]);
       }
     }
 #pragma unroll
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
             }
           }
         }
-        store_stream(&out[g], r, nt);
+        store_stream<NT>(&out[g], r);
       }
     }
   }
@@ -127,19 +127,16 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
-    if (t.flat_unroll >= 4) {
-      chan_map_kernel<f32x4, NIN, ACC, 4, Op>
-          <<<stream_grid(groups, 4), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
-    } else if (t.flat_unroll >= 2) {
-      chan_map_kernel<f32x4, NIN, ACC, 2, Op>
-          <<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
+    if (nt) {
+      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
     } else {
-      chan_map_kernel<f32x4, NIN, ACC, 1, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out, nt);
+      chan_map_kernel<f32x4, NIN, ACC, 1, 0, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
     }
   } else {
-    chan_map_kernel<float, NIN, ACC, 4, Op>
-        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out, 0);
+    chan_map_kernel<float, NIN, ACC, 4, 0, Op>
+        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out);
   }
   note_launch(symbol);
 }

@@ -69,12 +69,12 @@ __device__ inline void chan_reduce_term(const Op &op, const P &prm, float a, flo
   }
 }
 
-template <typename Op, typename V>
+template <typename Op, typename V, int NT>
 __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
                                                                    const float *__restrict__ c3,
-                                                                   double *__restrict__ part, int policy) {
+                                                                   double *__restrict__ part) {
   constexpr int W = VecLanes<V>::n;
   constexpr int U = 4;
   __shared__ double lds[kBlock / kWave];
@@ -105,9 +105,9 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
       for (int u = 0; u < U; ++u) {
         const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
         if (j < LG) {
-          va[u] = load_stream(&pa[j], policy);
-          if (Op::NIN >= 2) vb[u] = load_stream(&pb[j], policy);
-          if (Op::NIN >= 3) vc[u] = load_stream(&pc[j], policy);
+          va[u] = load_stream<NT>(&pa[j]);
+          if (Op::NIN >= 2) vb[u] = load_stream<NT>(&pb[j]);
+          if (Op::NIN >= 3) vc[u] = load_stream<NT>(&pc[j]);
         }
       }
 #pragma unroll
@@ -143,12 +143,12 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
   }
 }
 
-template <typename Op, typename V>
+template <typename Op, typename V, int NT>
 __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl, FastDiv div_s, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
                                                                    const float *__restrict__ c3,
-                                                                   double *__restrict__ part, int policy) {
+                                                                   double *__restrict__ part) {
   constexpr int W = VecLanes<V>::n;
   constexpr int G = 16 / W;                       // position groups owned by a thread
   constexpr int STAGES = (Op::NIN >= 2) ? 1 : 2;  // samples loaded before any is consumed
@@ -191,9 +191,9 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
 #pragma unroll
         for (int i = 0; i < G; ++i) {
           if (valid[i]) {
-            va[sg][i] = load_stream(&pa[threadIdx.x + uint32_t(i) * kBlock], policy);
-            if (Op::NIN >= 2) vb[sg][i] = load_stream(&pb[threadIdx.x + uint32_t(i) * kBlock], policy);
-            if (Op::NIN >= 3) vc[sg][i] = load_stream(&pc[threadIdx.x + uint32_t(i) * kBlock], policy);
+            va[sg][i] = load_stream<NT>(&pa[threadIdx.x + uint32_t(i) * kBlock]);
+            if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[threadIdx.x + uint32_t(i) * kBlock]);
+            if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[threadIdx.x + uint32_t(i) * kBlock]);
           }
         }
       }
@@ -302,15 +302,23 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
   if (pl.whole) {
     const FastDiv div_s(S);
     if (pl.vec) {
-      chan_reduce_whole_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part, nt);
+      if (nt) {
+        chan_reduce_whole_kernel<Op, f32x4, kNtLoad><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+      } else {
+        chan_reduce_whole_kernel<Op, f32x4, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+      }
     } else {
-      chan_reduce_whole_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part, nt);
+      chan_reduce_whole_kernel<Op, float, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
     }
   } else {
     if (pl.vec) {
-      chan_reduce_chunk_kernel<Op, f32x4><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part, nt);
+      if (nt) {
+        chan_reduce_chunk_kernel<Op, f32x4, kNtLoad><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part);
+      } else {
+        chan_reduce_chunk_kernel<Op, f32x4, 0><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part);
+      }
     } else {
-      chan_reduce_chunk_kernel<Op, float><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part, nt);
+      chan_reduce_chunk_kernel<Op, float, 0><<<pl.grid, kBlock, 0, s>>>(pl, op, a, b, c, part);
     }
   }
   note_launch(symbol);

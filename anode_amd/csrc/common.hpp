@@ -70,19 +70,26 @@ struct FastDiv {
 // ---------------------------------------------------------------------------
 #if defined(__HIPCC__)
 
-// Streaming accesses.  Bit 0 of `nt` marks stores, bit 1 marks loads as
+// Streaming accesses.  Bit 0 of NT marks stores, bit 1 marks loads as
 // non-temporal (the `nt` cache policy of global_load/global_store): the data is
-// touched once, so it should not displace reusable lines.
+// touched once, so it should not displace reusable lines.  NT is a template
+// parameter on purpose: a run-time choice between an ordinary and a
+// non-temporal access to the same address is folded into one ordinary access
+// by the compiler.
 constexpr int kNtStore = 1, kNtLoad = 2;
 
-template <typename V>
-__device__ inline V load_stream(const V *p, int nt) {
-  return (nt & kNtLoad) ? __builtin_nontemporal_load(p) : *p;
+template <int NT, typename V>
+__device__ inline V load_stream(const V *p) {
+  if constexpr ((NT & kNtLoad) != 0) {
+    return __builtin_nontemporal_load(p);
+  } else {
+    return *p;
+  }
 }
 
-template <typename V>
-__device__ inline void store_stream(V *p, V v, int nt) {
-  if (nt & kNtStore) {
+template <int NT, typename V>
+__device__ inline void store_stream(V *p, V v) {
+  if constexpr ((NT & kNtStore) != 0) {
     __builtin_nontemporal_store(v, p);
   } else {
     *p = v;
@@ -143,8 +150,8 @@ int device_cu_count();
 // Tunable launch parameters; defaults are set in runtime.hip and may be
 // changed at run time through anode_gpu_set_tuning().
 struct Tuning {
-  int flat_wg_per_cu;     // workgroups per CU of a streaming map; 0 = one trip per workgroup (full grid)
-  int flat_unroll;        // independent 16-byte groups per thread and loop trip (1, 2, 4 or 8)
+  int flat_wg_per_cu;     // workgroups per CU of a streaming map; 0 = one 16-byte group per thread (full grid)
+  int flat_unroll;        // unused (kept so that knob numbers stay stable)
   int reduce_wg_target;   // workgroups a per-channel reduction aims to launch
   int nontemporal;        // bit 0: non-temporal stores, bit 1: non-temporal loads (streaming maps)
   int reduce_nontemporal; // bit 1: non-temporal loads in the reductions

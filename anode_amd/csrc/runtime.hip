@@ -29,8 +29,8 @@ Tuning g_tuning = {
     /*flat_wg_per_cu=*/0,
     /*flat_unroll=*/1,
     /*reduce_wg_target=*/8192,
-    /*nontemporal=*/0,
-    /*reduce_nontemporal=*/0,
+    /*nontemporal=*/3,
+    /*reduce_nontemporal=*/2,
     /*nt_min_bytes=*/192 << 20,
 };
 

@@ -243,7 +243,7 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
 // multiplies by one correctly rounded reciprocal per pixel.  With NLL the
 // label gather is fused: nll = -log(the stored probability of the label), NaN
 // when the label is out of range, exactly what the separate gather returns.
-template <int CMAX, typename V, bool NLL>
+template <int CMAX, typename V, bool NLL, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 const uint32_t *__restrict__ cat,
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
 #pragma unroll
     for (int k = 0; k < CMAX; ++k) {
       if (uint32_t(k) < pg.C) {
-        v[k] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * k);
+        v[k] = load_stream<NT>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
         m = vmax(m, v[k]);
       }
     }
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     for (int k = 0; k < CMAX; ++k) {
       if (uint32_t(k) < pg.C) {
         const V pr = v[k] * inv;
-        *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = pr;
+        store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), pr);
         if (NLL) {
 #pragma unroll
           for (int w = 0; w < W; ++w) {
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
 
 // softmax.cu:315-334: dx[p,k,n] (=|+=) dy[p,n] * (prob - float(label[p,n]==k)).
 // A thread reads dy and the label of its pixels once and walks the classes.
-template <typename V, bool ACC>
+template <typename V, bool ACC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGrid pg,
                                                                         const float *__restrict__ dy,
                                                                         const float *__restrict__ prob,
@@ -373,16 +373,16 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
 #pragma unroll 4
     for (uint32_t k = 0; k < pg.C; ++k) {
       const size_t off = base + size_t(pg.P) * k;
-      const V pr = *reinterpret_cast<const V *>(prob + off);
+      const V pr = load_stream<NT>(reinterpret_cast<const V *>(prob + off));
       V old;
-      if (ACC) old = *reinterpret_cast<const V *>(dx + off);
+      if (ACC) old = load_stream<NT>(reinterpret_cast<const V *>(dx + off));
       V r;
 #pragma unroll
       for (int w = 0; w < W; ++w) {
         const float t = lane_get<V>(pr, w) - float(lane_get_u(lab, w) == k);
         lane_set<V>(r, w, ACC ? fmaf(lane_get<V>(d, w), t, lane_get<V>(old, w)) : lane_get<V>(d, w) * t);
       }
-      *reinterpret_cast<V *>(dx + off) = r;
+      store_stream<NT>(reinterpret_cast<V *>(dx + off), r);
     }
   }
 }
@@ -402,21 +402,34 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W) {
 uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
 // C <= 32 only
-template <typename V, bool NLL>
-void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
-                           float *nll, hipStream_t s) {
+template <typename V, bool NLL, int NT>
+void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
+                              float *nll, hipStream_t s) {
   const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
   const uint32_t blocks = pixel_blocks(pg.total_groups);
   if (C <= 4) {
-    softmax_nd_reg_kernel<4, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<4, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 8) {
-    softmax_nd_reg_kernel<8, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<8, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 16) {
-    softmax_nd_reg_kernel<16, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<16, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 24) {
-    softmax_nd_reg_kernel<24, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<24, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else {
-    softmax_nd_reg_kernel<32, V, NLL><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<32, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+  }
+}
+
+template <typename V, bool NLL>
+void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
+                           float *nll, hipStream_t s) {
+  // the input is streamed; the probabilities are read again by the NLL gather and the backward pass, so they
+  // keep the default policy unless they are far larger than the last-level cache
+  const size_t bytes = size_t(P) * C * N * sizeof(float);
+  if (PixVec<V>::W == 4 && stream_policy(bytes, tuning().nontemporal)) {
+    launch_softmax_nd_reg_nt<V, NLL, kNtLoad | kNtStore>(P, C, N, x, y, cat, nll, s);
+  } else {
+    launch_softmax_nd_reg_nt<V, NLL, 0>(P, C, N, x, y, cat, nll, s);
   }
 }
 
@@ -446,9 +459,9 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
     const uint32_t blocks = pixel_blocks(pg.total_groups);
     if (C <= 64) {
-      softmax_nd_reg_kernel<64, float, false><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      softmax_nd_reg_kernel<64, float, false, 0><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     } else {
-      softmax_nd_reg_kernel<128, float, false><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      softmax_nd_reg_kernel<128, float, false, 0><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     }
   } else if (vec) {
     launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
@@ -477,10 +490,15 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   if (vec) {
     const PixelGrid pg = make_pixel_grid(P, C, N, 4);
-    softmax_nd_cat_nll_bwd_kernel<f32x4, ACC><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+    if (stream_policy(size_t(len) * sizeof(float), tuning().nontemporal)) {
+      softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, kNtLoad | kNtStore>
+          <<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+    } else {
+      softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+    }
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
-    softmax_nd_cat_nll_bwd_kernel<float, ACC><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+    softmax_nd_cat_nll_bwd_kernel<float, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
   }
   note_launch(symbol);
 }
