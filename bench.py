@@ -35,6 +35,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated group names to run (default: all)")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="instead of the benchmark: time the library's plain copy and a read-only reduction on cold "
+                         "822 MB arrays under the launch-geometry and cache-policy knobs, one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="add one plain copy of a known size to the step (scale for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
@@ -45,6 +48,16 @@ class Launch:
 
     def __init__(self, group, symbol, args, alg_bytes, elements):
         self.group, self.symbol, self.args, self.alg_bytes, self.elements = group, symbol, args, alg_bytes, elements
+
+
+# HBM bytes per launch from hardware counters, keyed by (symbol, workload group): two rocprofv3 --pmc runs of this
+# file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy
+# of known size in the same run (--copy-calibration): FETCH_SIZE x 2.000, WRITE_SIZE x 0.998.  A launch that is not
+# listed reports null.
+MEASURED_TRAFFIC = {
+    # 802 838 KiB fetched, 802 816 KiB written; algorithmic bytes are 2 466 250 752
+    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2a"): 2465012000,
+}
 
 
 def build_workload(torch, only, copy_calibration=False):
@@ -162,6 +175,43 @@ def build_workload(torch, only, copy_calibration=False):
     return launches, fused
 
 
+def stream_probe(torch, gpu):
+    """The two measurements behind the launch geometry and the cache policy of the streaming kernels."""
+    n = 205520896  # 822 MB of f32
+    pairs = [(torch.randn(n, device="cuda"), torch.empty(n, device="cuda")) for _ in range(4)]  # rotate: cold data
+    S, C, N = 12544, 64, 256
+    mean = torch.empty(C, device="cuda")
+
+    def rate(fn, nbytes, reps=12):
+        for i in range(2):
+            fn(i)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(reps):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return round(nbytes / (a.elapsed_time(b) * 1e-3 / reps) / 1e9, 1)
+
+    saved = [gpu.set_tuning(k, -1) for k in range(6)]
+    out = {"bytes_per_array": 4 * n, "copy_gbps": {}, "batch_mean_gbps": {}}
+    gpu.set_tuning(5, 0)
+    for wg in (0, 8, 32):
+        for nt in (0, 3):
+            gpu.set_tuning(0, wg)
+            gpu.set_tuning(3, nt)
+            key = f"{'full_grid' if wg == 0 else str(wg) + '_wg_per_cu'}_{'nontemporal' if nt else 'default'}"
+            out["copy_gbps"][key] = rate(lambda i: gpu.call("anode_gpu_copy_flat_map_f32", n, *pairs[i % 4]), 8 * n)
+    for rnt in (0, 2):
+        gpu.set_tuning(4, rnt)
+        key = "nontemporal" if rnt else "default"
+        out["batch_mean_gbps"][key] = rate(
+            lambda i: gpu.call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, pairs[i % 4][0], mean), 4 * n)
+    for k, v in enumerate(saved):
+        gpu.set_tuning(k, v)
+    return out
+
+
 def cpu_baseline():
     """The fp32 CPU restatement (reference operation order) on a bounded sample of the same workload."""
     import numpy as np
@@ -249,6 +299,9 @@ def main():
         sys.stderr.write("bench.py: no GPU visible\n")
         sys.exit(3)
     torch.cuda.set_device(0)
+    if args.stream_probe:
+        print(json.dumps({"stream_probe": stream_probe(torch, gpu)}), flush=True)
+        return
     only = set(filter(None, args.only.split(",")))
     launches, fused = build_workload(torch, only, args.copy_calibration)
     torch.cuda.synchronize()
@@ -312,7 +365,7 @@ def main():
         "frac": round(dom.alg_bytes / dom_s / 1e9 / HBM_PEAK_GBPS, 4),
         "alg_bytes_per_launch": dom.alg_bytes,
         "avg_launch_us": round(dom_s * 1e6, 2),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC.get((dom.symbol, dom.group)),
     }
 
     groups = {}
