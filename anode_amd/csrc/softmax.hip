@@ -172,21 +172,28 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
 __global__ __launch_bounds__(kBlock) void softmax_cat_nll_kernel(uint32_t K, uint32_t R,
                                                                  const float *__restrict__ p,
                                                                  const uint32_t *__restrict__ cat,
-                                                                 float *__restrict__ nll) {
+                                                                 float *__restrict__ nll, bool ignore) {
   const uint32_t stride = gridDim.x * kBlock;
   for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < R; i += stride) {
     const uint32_t k = cat[i];
-    nll[i] = (k < K) ? -logf(p[size_t(k) + size_t(K) * i]) : __builtin_nanf("");
+    nll[i] = (k < K) ? -logf(p[size_t(k) + size_t(K) * i]) : (ignore ? 0.0f : __builtin_nanf(""));
   }
 }
 
 // softmax.cu:177-195  dx[k,i] (=|+=) dy[i] * (p[k,i] - float(label[i]==k)); as a
 // channel-indexed map the "channel" is the row i and s is the class k.
+// With ignore set, a row whose label is >= n_classes gets dy = 0 (the "ignore" variants); the reference's
+// semantics leaves the gradient unmasked.
 struct CatNllBwdMap {
   const float *dy;
   const uint32_t *cat;
+  uint32_t n_classes;
+  bool ignore;
   struct Param { float dy; uint32_t label; };
-  __device__ Param load(uint32_t i) const { return Param{dy[i], cat[i]}; }
+  __device__ Param load(uint32_t i) const {
+    const uint32_t label = cat[i];
+    return Param{(ignore && label >= n_classes) ? 0.0f : dy[i], label};
+  }
   __device__ float value(const Param &p, float prob, float, uint32_t k) const {
     return p.dy * (prob - float(p.label == k));
   }
@@ -228,6 +235,7 @@ __device__ inline f32x4 vrcp(f32x4 a) { return f32x4{1.0f / a.x, 1.0f / a.y, 1.0
 struct PixelGrid {
   uint32_t P, C, N;
   uint32_t total_groups;
+  uint32_t ignore;  // 1: an out-of-range label gives nll = 0 and no gradient, instead of NaN and dy * p
   FastDiv div_gps;  // groups per sample
 };
 
@@ -293,7 +301,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
       V out;
 #pragma unroll
       for (int w = 0; w < W; ++w) {
-        lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(lane_get<V>(picked, w)) : __builtin_nanf(""));
+        lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(lane_get<V>(picked, w))
+                                                      : (pg.ignore ? 0.0f : __builtin_nanf("")));
       }
       *reinterpret_cast<V *>(nll + (size_t(p) + size_t(pg.P) * n)) = out;
     }
@@ -346,7 +355,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
     V out;
 #pragma unroll
     for (int w = 0; w < W; ++w) {
-      lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr[w]) : __builtin_nanf(""));
+      lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr[w]) : (pg.ignore ? 0.0f : __builtin_nanf("")));
     }
     *reinterpret_cast<V *>(nll + pix) = out;
   }
@@ -368,8 +377,14 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
     pixel_decode(pg, g, W, p, n);
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
-    const V d = *reinterpret_cast<const V *>(dy + pix);
+    V d = *reinterpret_cast<const V *>(dy + pix);
     const U lab = *reinterpret_cast<const U *>(cat + pix);
+    if (pg.ignore) {
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        if (lane_get_u(lab, w) >= pg.C) lane_set<V>(d, w, 0.0f);
+      }
+    }
 #pragma unroll 4
     for (uint32_t k = 0; k < pg.C; ++k) {
       const size_t off = base + size_t(pg.P) * k;
@@ -387,8 +402,9 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
   }
 }
 
-PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W) {
+PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore = false) {
   PixelGrid pg;
+  pg.ignore = ignore ? 1u : 0u;
   pg.P = P;
   pg.C = C;
   pg.N = N;
@@ -473,23 +489,46 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
 
 template <bool ACC>
 void launch_softmax_cat_nll_bwd(const char *symbol, uint32_t K, uint32_t R, const float *dy, const float *prob,
-                                const uint32_t *cat, float *dx, CUstream_st *stream) {
-  launch_chan_map<1, ACC>(symbol, K, R, 1, CatNllBwdMap{dy, cat}, prob, nullptr, dx, stream);
+                                const uint32_t *cat, float *dx, CUstream_st *stream, bool ignore = false) {
+  launch_chan_map<1, ACC>(symbol, K, R, 1, CatNllBwdMap{dy, cat, K, ignore}, prob, nullptr, dx, stream);
+}
+
+void launch_softmax_cat_nll(const char *symbol, uint32_t K, uint32_t R, const float *prob, const uint32_t *cat,
+                            float *nll, CUstream_st *stream, bool ignore) {
+  (void)checked_len(K, R, 1, symbol);
+  if (R == 0) return;
+  softmax_cat_nll_kernel<<<stream_grid(R, 1), kBlock, 0, as_stream(stream)>>>(K, R, prob, cat, nll, ignore);
+  note_launch(symbol);
+}
+
+void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *prob,
+                               const uint32_t *cat, float *nll, CUstream_st *stream, bool ignore) {
+  (void)checked_len(P, C, N, symbol);
+  if (P == 0 || N == 0) return;
+  if (P % 4 == 0 && aligned16(cat) && aligned16(nll)) {
+    const PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
+    softmax_nd_cat_nll_kernel<f32x4><<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, prob, cat, nll);
+  } else {
+    const PixelGrid pg = make_pixel_grid(P, C, N, 1, ignore);
+    softmax_nd_cat_nll_kernel<float><<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, prob, cat, nll);
+  }
+  note_launch(symbol);
 }
 
 template <bool ACC>
 void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *dy,
-                                   const float *prob, const uint32_t *cat, float *dx, CUstream_st *stream) {
+                                   const float *prob, const uint32_t *cat, float *dx, CUstream_st *stream,
+                                   bool ignore = false) {
   const uint32_t len = checked_len(P, C, N, symbol);
   if (len == 0) return;
   if (P == 1) {
-    launch_softmax_cat_nll_bwd<ACC>(symbol, C, N, dy, prob, cat, dx, stream);
+    launch_softmax_cat_nll_bwd<ACC>(symbol, C, N, dy, prob, cat, dx, stream, ignore);
     return;
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   if (vec) {
-    const PixelGrid pg = make_pixel_grid(P, C, N, 4);
+    const PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
     if (stream_policy(size_t(len) * sizeof(float), tuning().nontemporal)) {
       softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, kNtLoad | kNtStore>
           <<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
@@ -497,7 +536,7 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
       softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
     }
   } else {
-    const PixelGrid pg = make_pixel_grid(P, C, N, 1);
+    const PixelGrid pg = make_pixel_grid(P, C, N, 1, ignore);
     softmax_nd_cat_nll_bwd_kernel<float, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
   }
   note_launch(symbol);
@@ -522,10 +561,7 @@ ANODE_EXPORT void anode_gpu_softmax_packed_deterministic_f32(uint32_t dim0, uint
 ANODE_EXPORT void anode_gpu_softmax_cat_nll_packed_f32(uint32_t dim0, uint32_t dim1, const float *softmax,
                                                        const uint32_t *cat_data, float *nll,
                                                        const KernelConfig *, CUstream_st *stream) {
-  (void)checked_len(dim0, dim1, 1, __func__);
-  if (dim1 == 0) return;
-  softmax_cat_nll_kernel<<<stream_grid(dim1, 1), kBlock, 0, as_stream(stream)>>>(dim0, dim1, softmax, cat_data, nll);
-  note_launch(__func__);
+  launch_softmax_cat_nll(__func__, dim0, dim1, softmax, cat_data, nll, stream, false);
 }
 
 ANODE_EXPORT void anode_gpu_softmax_cat_nll_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy,
@@ -550,18 +586,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_packed_f32(uint32_t prefix_dim, uint32_t 
 ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
                                                           const float *softmax, const uint32_t *cat_data,
                                                           float *nll, const KernelConfig *, CUstream_st *stream) {
-  (void)checked_len(prefix_dim, dim0, dim1, __func__);
-  if (prefix_dim == 0 || dim1 == 0) return;
-  if (prefix_dim % 4 == 0 && aligned16(cat_data) && aligned16(nll)) {
-    const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 4);
-    softmax_nd_cat_nll_kernel<f32x4>
-        <<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
-  } else {
-    const PixelGrid pg = make_pixel_grid(prefix_dim, dim0, dim1, 1);
-    softmax_nd_cat_nll_kernel<float>
-        <<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, softmax, cat_data, nll);
-  }
-  note_launch(__func__);
+  launch_softmax_nd_cat_nll(__func__, prefix_dim, dim0, dim1, softmax, cat_data, nll, stream, false);
 }
 
 ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
@@ -602,4 +627,52 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
     anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
   }
+}
+
+// Additive "ignore" variants (no counterpart in the reference, whose kernels give NaN and an unmasked gradient for
+// a label >= the number of classes, softmax.cu:294-296, :331): such a row or pixel contributes nll = 0 and dx = 0
+// (for _accumulate: dx unchanged).  In-range labels give bit-identical results to the plain entry points.
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_ignore_packed_f32(uint32_t dim0, uint32_t dim1, const float *softmax,
+                                                              const uint32_t *cat_data, float *nll,
+                                                              const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_cat_nll(__func__, dim0, dim1, softmax, cat_data, nll, stream, true);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_bwd_ignore_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy,
+                                                                  const float *softmax, const uint32_t *cat_data,
+                                                                  float *dx, const KernelConfig *,
+                                                                  CUstream_st *stream) {
+  launch_softmax_cat_nll_bwd<false>(__func__, dim0, dim1, dy, softmax, cat_data, dx, stream, true);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_bwd_ignore_packed_accumulate_f32(uint32_t dim0, uint32_t dim1,
+                                                                             const float *dy, const float *softmax,
+                                                                             const uint32_t *cat_data, float *dx,
+                                                                             const KernelConfig *,
+                                                                             CUstream_st *stream) {
+  launch_softmax_cat_nll_bwd<true>(__func__, dim0, dim1, dy, softmax, cat_data, dx, stream, true);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_ignore_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
+                                                                 const float *softmax, const uint32_t *cat_data,
+                                                                 float *nll, const KernelConfig *,
+                                                                 CUstream_st *stream) {
+  launch_softmax_nd_cat_nll(__func__, prefix_dim, dim0, dim1, softmax, cat_data, nll, stream, true);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_ignore_packed_f32(uint32_t prefix_dim, uint32_t dim0,
+                                                                     uint32_t dim1, const float *dy,
+                                                                     const float *softmax, const uint32_t *cat_data,
+                                                                     float *dx, const KernelConfig *,
+                                                                     CUstream_st *stream) {
+  launch_softmax_nd_cat_nll_bwd<false>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream, true);
+}
+
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_ignore_packed_accumulate_f32(uint32_t prefix_dim, uint32_t dim0,
+                                                                                uint32_t dim1, const float *dy,
+                                                                                const float *softmax,
+                                                                                const uint32_t *cat_data, float *dx,
+                                                                                const KernelConfig *,
+                                                                                CUstream_st *stream) {
+  launch_softmax_nd_cat_nll_bwd<true>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream, true);
 }

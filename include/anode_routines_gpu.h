@@ -227,6 +227,41 @@ void anode_gpu_online_average_packed_f32(uint32_t len, float rate, const float *
  * strict maximum, NaN never selected, 0 when nothing exceeds -inf. */
 void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, const float *x, uint32_t *index, ANODE_LAUNCH_TAIL);
 
+/* "Ignore" variants of the four NLL entry points above: a label >= the number of classes contributes nll = 0 and
+ * dx = 0 (dx unchanged for _accumulate) instead of the reference's NaN and unmasked dy*p (softmax.cu:294-296, :331).
+ * In-range labels give bit-identical results to the plain entry points. */
+void anode_gpu_softmax_cat_nll_ignore_packed_f32(uint32_t dim0, uint32_t dim1, const float *softmax, const uint32_t *cat_data, float *nll, ANODE_LAUNCH_TAIL);
+void anode_gpu_softmax_cat_nll_bwd_ignore_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+void anode_gpu_softmax_cat_nll_bwd_ignore_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+void anode_gpu_softmax_nd_cat_nll_ignore_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *softmax, const uint32_t *cat_data, float *nll, ANODE_LAUNCH_TAIL);
+void anode_gpu_softmax_nd_cat_nll_bwd_ignore_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+void anode_gpu_softmax_nd_cat_nll_bwd_ignore_packed_accumulate_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
+
+/* ---- the neighbours anode takes from its sibling library gpudevicemem (source not part of the reference tree) ----
+ * Signatures follow the call sites in src/ops_gpu.rs; the arithmetic is the closed form those call sites imply.
+ * Exported under this library's prefix so that both libraries can be linked together. */
+
+/* src/ops_gpu.rs:7486-7492 (gpudevicemem_sum_packed_deterministic_f32): y[0] = sum_i x[i]; fp64 accumulation in a fixed order. */
+void anode_gpu_sum_packed_deterministic_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7499-7505.  y[0] += sum_i x[i] */
+void anode_gpu_sum_packed_accumulate_deterministic_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7595-7601 (gpudevicemem_bcast_packed_f32): y[i] = x[0] for i < len; x is a device scalar. */
+void anode_gpu_bcast_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7608-7614.  y[i] += x[0] */
+void anode_gpu_bcast_packed_accumulate_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:9592-9600 (gpudevicemem_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32): y[a,b] = x[a,b] / rdivisor[b]. */
+void anode_gpu_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32(uint32_t inner_dim, uint32_t outer_dim, const float *x, const float *rdivisor, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:1244, :2080 (set_zeros, set_constant): y[i] = c. */
+void anode_gpu_set_constant_packed_f32(uint32_t len, float c, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:108, :557 (add): y[i] += x[i].  (copy is anode_gpu_copy_flat_map_f32.) */
+void anode_gpu_add_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:3346 (mult): y[i] *= x[i]. */
+void anode_gpu_mult_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:3636 (is_nonzero): y[i] = float(x[i] != 0). */
+void anode_gpu_is_nonzero_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:5886 (online_add): y[i] = fma(rate, x[i], y[i]). */
+void anode_gpu_online_add_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
+
 /* The host-side rule itself (src/utils/mod.rs:31-41), for logits already on the host: first index of the strict
  * maximum starting from (-inf, 0); NaN never selected.  xs is a HOST pointer. */
 size_t anode_host_arg_max_f32(const float *xs, size_t len);

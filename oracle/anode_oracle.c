@@ -905,3 +905,29 @@ ORACLE_API void oracle_batch_norm_affine_f64(uint32_t d0, uint32_t d1, uint32_t 
 ORACLE_API void oracle_online_average(uint32_t len, float rate, const float *x, float *y) {
   for (uint32_t i = 0; i < len; ++i) y[i] = fmaf(rate, x[i] - y[i], y[i]);
 }
+
+/* --------------------------------------------------------------------------
+ * The neighbours anode takes from gpudevicemem (no source in the reference
+ * tree): closed forms implied by the call sites in src/ops_gpu.rs.
+ * Parity unpinned by the reference except for the fills and the sum-join
+ * value of tests/test_gpu.rs:245-353.
+ * -------------------------------------------------------------------------- */
+
+/* src/ops_gpu.rs:7486: y = sum_i x[i], here as the fp64 sum */
+ORACLE_API double oracle_sum_packed_f64(uint32_t len, const float *x) {
+  double s = 0.0;
+  for (uint32_t i = 0; i < len; ++i) s += (double)x[i];
+  return s;
+}
+
+/* src/ops_gpu.rs:5886: y <- y + rate * x, one fmaf */
+ORACLE_API void oracle_online_add(uint32_t len, float rate, const float *x, float *y) {
+  for (uint32_t i = 0; i < len; ++i) y[i] = fmaf(rate, x[i], y[i]);
+}
+
+/* src/ops_gpu.rs:9592: y[a,b] = x[a,b] / r[b], IEEE division */
+ORACLE_API void oracle_flat_bcast_rdiv(uint32_t inner, uint32_t outer, const float *x, const float *r,
+                                       float *y) {
+  for (uint32_t b = 0; b < outer; ++b)
+    for (uint32_t a = 0; a < inner; ++a) y[a + (size_t)inner * b] = x[a + (size_t)inner * b] / r[b];
+}

@@ -420,3 +420,28 @@ def batch_norm_affine(d0, d1, d2, x, mean, var, gamma, beta, f64=False):
     fn = lib().oracle_batch_norm_affine_f64 if f64 else lib().oracle_batch_norm_affine_f32ref
     fn(u32(d0), u32(d1), u32(d2), _p(x), _p(mean), _p(var), _p(gamma), _p(beta), _p(out))
     return out
+
+
+# --------------------------------------------------------------------------
+# neighbours from gpudevicemem (closed forms of the call sites)
+# --------------------------------------------------------------------------
+
+def sum_packed(x) -> float:
+    x = _f32(x).ravel()
+    fn = lib().oracle_sum_packed_f64
+    fn.restype = ctypes.c_double
+    return float(fn(u32(x.size), _p(x)))
+
+
+def online_add(rate, x, y):
+    x = _f32(x).ravel()
+    out = _f32(y).ravel().copy()
+    lib().oracle_online_add(u32(x.size), f32(rate), _p(x), _p(out))
+    return out
+
+
+def flat_bcast_rdiv(inner, outer, x, r):
+    x, r = _f32(x).ravel(), _f32(r).ravel()
+    out = np.empty(inner * outer, np.float32)
+    lib().oracle_flat_bcast_rdiv(u32(inner), u32(outer), _p(x), _p(r), _p(out))
+    return out
