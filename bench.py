@@ -212,6 +212,72 @@ def stream_probe(torch, gpu):
     return out
 
 
+def small_shape_latency(torch, gpu, groups, passes=100):
+    """Launch-bound shapes (config 0, config 3a): time per pass over `passes` back-to-back passes, launched one entry
+    point at a time and as one captured HIP graph replayed.  Separates launch latency from bandwidth."""
+    out = {}
+    stream = torch.cuda.Stream()
+    for name, ls in groups.items():
+        def run():
+            for l in ls:
+                gpu.call(l.symbol, *l.args)
+        with torch.cuda.stream(stream):
+            run()  # allocates the reductions' scratch for this stream before anything is captured
+            run()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            run()
+        times = {}
+        for kind, once in (("eager", run), ("graph", graph.replay)):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with torch.cuda.stream(stream):
+                once()
+                a.record()
+                for _ in range(passes):
+                    once()
+                b.record()
+            stream.synchronize()
+            times[kind] = a.elapsed_time(b) * 1e-3 / passes
+        nbytes = sum(l.alg_bytes for l in ls)
+        out[name] = {"launches": len(ls), "eager_us_per_pass": round(times["eager"] * 1e6, 2),
+                     "graph_us_per_pass": round(times["graph"] * 1e6, 2),
+                     "graph_gbps": round(nbytes / times["graph"] / 1e9, 1)}
+    return out
+
+
+def small_shape_groups(torch, launches):
+    """Config 0 (BN on [32,16,28,28], softmax + NLL on [32,10]) and the config 3a launches of the step."""
+    def empty(n):
+        return torch.empty(n, device="cuda")
+    S, C, N = 784, 16, 32
+    n = S * C * N
+    x, dy, y, dx = torch.randn(n, device="cuda"), torch.randn(n, device="cuda"), empty(n), empty(n)
+    m, v, dm, dv = empty(C), empty(C), empty(C), empty(C)
+    d = (S, C, N)
+    bn0 = [Launch("bn_cfg0", "anode_gpu_batch_mean_3d1_packed_f32", (*d, x, m), 4 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_var_3d1_packed_f32", (*d, 1e-5, x, m, v), 4 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_norm_3d1_packed_f32", (*d, x, m, v, y), 8 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_norm_bwd_3d1_packed_f32", (*d, dy, v, dx), 8 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_norm_bwd_mean_3d1_packed_f32", (*d, dy, v, dm), 4 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_norm_bwd_var_3d1_packed_f32", (*d, dy, x, m, v, dv), 8 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", (*d, dv, x, m, dx), 12 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_var_bwd_mean_3d1_packed_accumulate_f32", (*d, dv, x, m, dm), 4 * n, n),
+           Launch("bn_cfg0", "anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32", (*d, dm, dx), 8 * n, n)]
+    K, R = 10, 32
+    lg, p, nll, dl = torch.randn(K * R, device="cuda"), empty(K * R), empty(R), empty(K * R)
+    lab = torch.randint(0, K, (R,), device="cuda", dtype=torch.int32)
+    ones = torch.ones(R, device="cuda")
+    sm0 = [Launch("softmax_cfg0", "anode_gpu_softmax_packed_block_f32", (K, R, lg, p), 8 * K * R, K * R),
+           Launch("softmax_cfg0", "anode_gpu_softmax_cat_nll_packed_f32", (K, R, p, lab, nll), 12 * R, R),
+           Launch("softmax_cfg0", "anode_gpu_softmax_cat_nll_bwd_packed_f32", (K, R, ones, p, lab, dl), 8 * K * R + 8 * R, K * R)]
+    groups = {"bn_fwd_bwd_cfg0": bn0, "softmax_nll_cfg0": sm0}
+    cfg3a = [l for l in launches if l.group == "softmax_cfg3a"]
+    if cfg3a:
+        groups["softmax_nll_cfg3a"] = cfg3a
+    return groups
+
+
 def cpu_baseline():
     """The fp32 CPU restatement (reference operation order) on a bounded sample of the same workload."""
     import numpy as np
@@ -273,10 +339,21 @@ def cpu_baseline():
     while passes < 16 and (passes == 0 or total_s < 1.5):
         one_pass()
         passes += 1
+    multi = (total_bytes, total_s, dict(parts), passes)
+    # the same sample once on one thread (the scalar figure beside the threaded one)
+    o.set_threads(1)
+    total_bytes, total_s = 0, 0.0
+    parts.clear()
+    one_pass()
+    single_gbps = total_bytes / total_s / 1e9
+    single_s = total_s
+    o.set_threads(threads)
+    total_bytes, total_s, parts, passes = multi
     return {
         "value": round(total_bytes / total_s / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "single_thread": {"value": round(single_gbps, 3), "unit": "GB/s", "cores": 1, "seconds": round(single_s, 2)},
         "kind": "port",
         "sample": "fp32 CPU restatement, OpenMP: BN fwd+bwd (9 launches) on [64,64,112,112]; softmax_nd+NLL+bwd on "
                   "[4,19,512,1024]; dequantize+upcast on [256,3,224,224]; repeated to ~1.5 s; algorithmic bytes / time",
@@ -447,6 +524,8 @@ def main():
         "fused_model": fused_model,
         "per_symbol": per_symbol,
     }
+    if not only:
+        out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)
