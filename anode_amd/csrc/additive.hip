@@ -31,8 +31,8 @@ __global__ __launch_bounds__(kBlock) void quantize_u8x4_kernel(uint32_t n_groups
                                                                uint8_t *__restrict__ y) {
   const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
   uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < n_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
     const f32x4 v = x4[g];
     y4[g] = quantize_one(v.x, lo, scale) | (quantize_one(v.y, lo, scale) << 8) |
             (quantize_one(v.z, lo, scale) << 16) | (quantize_one(v.w, lo, scale) << 24);
@@ -46,8 +46,8 @@ __global__ __launch_bounds__(kBlock) void quantize_u8x4_kernel(uint32_t n_groups
 __global__ __launch_bounds__(kBlock) void quantize_u8_scalar_kernel(uint32_t len, float lo, float scale,
                                                                     const float *__restrict__ x,
                                                                     uint8_t *__restrict__ y) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = uint8_t(quantize_one(x[i], lo, scale));
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) y[i] = uint8_t(quantize_one(x[i], lo, scale));
 }
 
 // ---------------------------------------------------------------------------
@@ -97,8 +97,8 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t 
   const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
   f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
   const uint32_t S = div_s.d, C = div_c.d;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < n_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
     const uint32_t w = x4[g];
     uint32_t q, s;
     div_s.divmod(g * 4u, q, s);
@@ -131,8 +131,8 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8_scalar_kernel(uint
                                                                             const float *__restrict__ shift,
                                                                             const uint8_t *__restrict__ x,
                                                                             float *__restrict__ y) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) {
     const uint32_t q = div_s.div(i);
     const uint32_t c = q - div_c.div(q) * div_c.d;
     y[i] = fmaf(scale[c], float(x[i]), shift[c]);
@@ -273,8 +273,8 @@ struct OnlineAverageMap {
 
 __global__ __launch_bounds__(kBlock) void online_average_kernel(uint32_t len, float rate,
                                                                 const float *__restrict__ x, float *y) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = fmaf(rate, x[i] - y[i], y[i]);
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) y[i] = fmaf(rate, x[i] - y[i], y[i]);
 }
 
 // First index of the strict maximum of each row of a [K (fastest), R] array;
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kBlock) void arg_max_rows_kernel(uint32_t K, uint32
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t n_waves = gridDim.x * (kBlock / kWave);
-  for (uint32_t r = wave; r < R; r += n_waves) {
+  for (uint64_t r = wave; r < R; r += n_waves) {
     const float *xr = x + size_t(r) * K;
     float top = -__builtin_huge_valf();
     uint32_t idx = 0xffffffffu;  // nothing above -inf seen yet

@@ -59,12 +59,12 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
   V *out = reinterpret_cast<V *>(out_);
   const uint32_t S = div_s.d, C = div_c.d;
   constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint32_t stride = gridDim.x * kTile;
-  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
     V va[UNROLL], vb[UNROLL], vc[UNROLL], vo[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
         if (NIN >= 1) va[u] = load_stream<NT>(&a[g]);
         if (NIN >= 2) vb[u] = load_stream<NT>(&b[g]);
@@ -74,10 +74,10 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
         uint32_t q, s;
-        div_s.divmod(g * uint32_t(L), q, s);
+        div_s.divmod(uint32_t(g) * uint32_t(L), q, s);
         uint32_t c = q - div_c.div(q) * C;
         typename Op::Param p = op.load(c);
         V r;

@@ -17,8 +17,8 @@ __global__ __launch_bounds__(kBlock) void one_hot_kernel(uint32_t P, uint32_t K,
                                                          float *__restrict__ y) {
   typedef typename std::conditional<W == 4, u32x4, uint32_t>::type U;
   typedef typename std::conditional<W == 4, f32x4, float>::type V;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < total_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < total_groups; g += stride) {
     uint32_t n, r;
     div_gps.divmod(g, n, r);
     const uint32_t p = r * uint32_t(W);

@@ -84,12 +84,12 @@ __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uin
   const V *b = reinterpret_cast<const V *>(b_);
   V *out = reinterpret_cast<V *>(out_);
   constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint32_t stride = gridDim.x * kTile;
-  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
     V va[UNROLL], vb[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
         va[u] = load_stream<NT>(&a[g]);
         vb[u] = (NIN == 2) ? load_stream<NT>(&b[g]) : va[u];
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uin
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) store_stream<NT>(&out[g], apply_vec(op, va[u], vb[u]));
     }
   }
@@ -156,17 +156,17 @@ __global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, u
   const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
   O4 *y4 = reinterpret_cast<O4 *>(y);
   constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint32_t stride = gridDim.x * kTile;
-  for (uint32_t base = blockIdx.x * kTile; base < n_groups; base += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
     uint32_t w[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) w[u] = load_stream<NT>(&x4[g]);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const uint32_t g = base + uint32_t(u) * kBlock + threadIdx.x;
+      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
       if (g < n_groups) {
         O4 r;
         r.x = op(w[u] & 0xffu);
@@ -187,8 +187,8 @@ template <typename Op>
 __global__ __launch_bounds__(kBlock) void widen_u8_scalar_kernel(uint32_t len, Op op,
                                                                  const uint8_t *__restrict__ x,
                                                                  typename Op::out_t *__restrict__ y) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) y[i] = op(uint32_t(x[i]));
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) y[i] = op(uint32_t(x[i]));
 }
 
 template <typename Op>

@@ -36,8 +36,8 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
   const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t n_waves = gridDim.x * (kBlock / kWave);
   // the loop bound depends on the wave only, so all 64 lanes reach every shuffle
-  for (uint32_t r0 = wave * rows_per_wave; r0 < R; r0 += n_waves * rows_per_wave) {
-    const uint32_t r = r0 + sub;
+  for (uint64_t r0 = uint64_t(wave) * rows_per_wave; r0 < R; r0 += uint64_t(n_waves) * rows_per_wave) {
+    const uint64_t r = r0 + sub;
     const bool valid = (k < K) && (r < R);
     const size_t idx = size_t(r) * K + k;
     const float v = valid ? x[idx] : kNegInf;
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t n_waves = gridDim.x * (kBlock / kWave);
-  for (uint32_t r = wave; r < R; r += n_waves) {
+  for (uint64_t r = wave; r < R; r += n_waves) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
     float v[VPL];
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
                                                                    const float *__restrict__ x,
                                                                    float *__restrict__ y) {
   __shared__ float lds_m[kBlock / kWave], lds_s[kBlock / kWave];
-  for (uint32_t r = blockIdx.x; r < R; r += gridDim.x) {
+  for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
     float m = kNegInf, s = 0.0f;
@@ -173,8 +173,8 @@ __global__ __launch_bounds__(kBlock) void softmax_cat_nll_kernel(uint32_t K, uin
                                                                  const float *__restrict__ p,
                                                                  const uint32_t *__restrict__ cat,
                                                                  float *__restrict__ nll, bool ignore) {
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < R; i += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < R; i += stride) {
     const uint32_t k = cat[i];
     nll[i] = (k < K) ? -logf(p[size_t(k) + size_t(K) * i]) : (ignore ? 0.0f : __builtin_nanf(""));
   }
@@ -258,8 +258,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
                                                                 float *__restrict__ nll) {
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
@@ -314,8 +314,8 @@ template <typename V>
 __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                    float *__restrict__ y) {
   constexpr int W = PixVec<V>::W;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
@@ -339,8 +339,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
                                                                     float *__restrict__ nll) {
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t pix = size_t(p) + size_t(pg.P) * n;
@@ -371,8 +371,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
                                                                         float *dx) {
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
-  const uint32_t stride = gridDim.x * kBlock;
-  for (uint32_t g = blockIdx.x * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t pix = size_t(p) + size_t(pg.P) * n;

@@ -1,7 +1,7 @@
 """Helpers shared by the GPU parity tests: device buffers, calls through the
 C ABI and the comparison bars.
 
-Bars (north-star of this build):
+Bars:
   * bit-exact for integer / byte / index work and for maps whose fp32
     arithmetic is fully specified (compare, multiply, correctly rounded
     divide and sqrt, the fused multiply-adds the reference's compiler forms);

@@ -1,0 +1,97 @@
+"""Arrays of more than 2^31 elements (the ABI's counts are 32-bit, so up to 2^32 - 1): every index computation in the
+kernels has to survive element offsets, and offset + grid stride, beyond 2^31 and close to 2^32.
+
+torch is the checker here (same formula on the device; a host copy of 8 GiB arrays would only add minutes): exact
+equality for the maps, 1e-5 against float64 for the reductions and the softmax.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import call
+
+pytestmark = pytest.mark.gpu
+
+N_BIG = (1 << 31) + (1 << 20) + 7   # odd, above 2^31
+
+
+@pytest.fixture(scope="module")
+def big():
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    x = torch.empty(N_BIG + 4, device="cuda")
+    x.normal_(generator=g)
+    yield x
+    del x
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("offset", [0, 1])
+def test_flat_map_beyond_2_31(big, offset):
+    x = big[offset:offset + N_BIG]
+    y = torch.full((N_BIG + 4,), float("nan"), device="cuda")
+    call("anode_gpu_positive_clip_flat_map_f32", N_BIG, x, y[offset:offset + N_BIG])
+    torch.cuda.synchronize()
+    assert torch.equal(y[offset:offset + N_BIG], torch.relu(x))
+    assert bool(torch.isnan(y[offset + N_BIG:]).all()) and bool(torch.isnan(y[:offset]).all())
+    del y
+
+
+@pytest.mark.parametrize("offset", [0, 1])
+def test_accumulate_map_applies_once_beyond_2_31(big, offset):
+    x = big[offset:offset + N_BIG]
+    y = torch.ones(N_BIG + 4, device="cuda")
+    call("anode_gpu_add_packed_f32", N_BIG, x, y[offset:offset + N_BIG])
+    torch.cuda.synchronize()
+    assert torch.equal(y[offset:offset + N_BIG], x + 1.0)
+    assert bool((y[offset + N_BIG:] == 1).all())
+    del y
+
+
+@pytest.mark.parametrize("offset", [0, 1])
+def test_batch_norm_pieces_beyond_2_31(big, offset):
+    S, C, N = 1 << 20, 3, 683           # 2 148 532 224 elements
+    n = S * C * N
+    assert (1 << 31) < n <= N_BIG
+    x = big[offset:offset + n]
+    mean, var = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, x, mean)
+    call("anode_gpu_batch_var_3d1_packed_f32", S, C, N, 1e-5, x, mean, var)
+    torch.cuda.synchronize()
+    xv = x.view(N, C, S)
+    for c in range(C):
+        col = xv[:, c, :].double()
+        m = col.mean().item()
+        v = ((col - float(mean[c])) ** 2).mean().item() + 1e-5
+        assert abs(float(mean[c]) - m) <= 1e-5 * abs(m) + 1e-7
+        assert abs(float(var[c]) - v) <= 1e-5 * v
+        del col
+    dx = torch.zeros(n + 4, device="cuda")[offset:offset + n]
+    dmean = torch.tensor([1.0, 2.0, 3.0], device="cuda") * float(S * N)
+    call("anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32", S, C, N, dmean, dx)
+    torch.cuda.synchronize()
+    want = torch.tensor([1.0, 2.0, 3.0], device="cuda").view(1, C, 1).expand(N, C, S)
+    assert torch.equal(dx.view(N, C, S), want)
+    del dx
+
+
+def test_softmax_nd_beyond_2_31(big):
+    P, C, N = 1 << 16, 19, 1725         # 2 147 942 400 elements
+    n = P * C * N
+    assert (1 << 31) < n <= N_BIG
+    x = big[:n]
+    p = torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_packed_f32", P, C, N, x, p)
+    lab = torch.randint(0, C, (P * N,), device="cuda", dtype=torch.int32)
+    nll = torch.empty(P * N, device="cuda")
+    call("anode_gpu_softmax_nd_cat_nll_packed_f32", P, C, N, p, lab, nll)
+    torch.cuda.synchronize()
+    pv = p.view(N, C, P)
+    for i in (0, N // 2, N - 1):        # float64 checks on single samples (the first, one across 2^31, the last)
+        ref = torch.softmax(x.view(N, C, P)[i].double(), dim=0)
+        assert bool(((pv[i].double() - ref).abs() <= 1e-5 * ref).all())
+        picked = torch.gather(pv[i], 0, lab.view(N, P)[i].long().unsqueeze(0)).squeeze(0)
+        assert torch.allclose(nll.view(N, P)[i], -torch.log(picked), rtol=1e-5, atol=1e-6)
+    sums = pv.sum(dim=1)
+    assert bool(((sums - 1).abs() < 1e-5).all())
+    del p, sums
