@@ -456,6 +456,80 @@ struct LeakyReluBwdOp {  // :8924
 };
 
 // ---------------------------------------------------------------------------
+// the neighbours the reference takes from gpudevicemem: batch sum / broadcast,
+// division by a per-sample scalar, running statistics, fills
+// ---------------------------------------------------------------------------
+
+struct BatchSumOp {  // src/ops_gpu.rs:7478-7505: x is a batch of scalars, y one scalar
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("BatchSumOp", x, y);
+    const uint32_t len = sz2uint(x.shape.flat_len());
+    if (cap == WriteCap::Assign) {
+      anode_gpu_sum_packed_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+    } else {
+      anode_gpu_sum_packed_accumulate_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+                                                        conn.cuda_stream());
+    }
+  }
+};
+
+struct BatchBroadcastOp {  // src/ops_gpu.rs:7585-7614 (and :7706-7719): x is one scalar, y a batch of scalars
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("BatchBroadcastOp", x, y);
+    const uint32_t len = sz2uint(y.shape.flat_len());
+    if (cap == WriteCap::Assign) {
+      anode_gpu_bcast_packed_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+    } else {
+      anode_gpu_bcast_packed_accumulate_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+    }
+  }
+};
+
+struct FlatBroadcastRdivOp {  // src/ops_gpu.rs:9575-9605: y[.., b] = x[.., b] / rdivisor[b]
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, const DeviceArray<float> &rdivisor,
+                    DeviceArray<float> &y) {
+    detail::require_packed("FlatBroadcastRdivOp", x, rdivisor, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("FlatBroadcastRdivOp: Accumulate");  // :9602
+    if (x.shape.batch != rdivisor.shape.batch) throw std::invalid_argument("FlatBroadcastRdivOp: batch sizes differ");  // :9578
+    const size_t batch = x.shape.batch;
+    anode_gpu_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32(sz2uint(batch ? x.shape.flat_len() / batch : 0), sz2uint(batch),
+                                                      x.as_dptr(), rdivisor.as_dptr(), y.as_mut_dptr(),
+                                                      conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct OnlineAverageOp {  // src/ops_gpu.rs:6059: y <- y + rate * (x - y), in place on y
+  static void apply(const GPUDeviceConn &conn, float rate, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("OnlineAverageOp", x, y);
+    anode_gpu_online_average_packed_f32(sz2uint(x.shape.flat_len()), rate, x.as_dptr(), y.as_mut_dptr(),
+                                        conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct OnlineAddOp {  // src/ops_gpu.rs:5886, :5929: y <- y + rate * x, in place on y
+  static void apply(const GPUDeviceConn &conn, float rate, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("OnlineAddOp", x, y);
+    anode_gpu_online_add_packed_f32(sz2uint(x.shape.flat_len()), rate, x.as_dptr(), y.as_mut_dptr(),
+                                    conn.cuda_kernel_config(), conn.cuda_stream());
+  }
+};
+
+struct IsNonzeroOp {  // src/ops_gpu.rs:3620-3640
+  static void apply(WriteCap cap, const GPUDeviceConn &conn, const DeviceArray<float> &x, DeviceArray<float> &y) {
+    detail::require_packed("IsNonzeroOp", x, y);
+    if (cap != WriteCap::Assign) throw Unimplemented("IsNonzeroOp: Accumulate");  // :3639
+    anode_gpu_is_nonzero_packed_f32(sz2uint(x.shape.flat_len()), x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+                                    conn.cuda_stream());
+  }
+};
+
+// zeros() / ones() sources (src/ops_gpu.rs:1244, :2080): Assign fills, Accumulate of zeros is a no-op and of ones adds 1
+inline void set_constant(const GPUDeviceConn &conn, float c, DeviceArray<float> &y) {
+  detail::require_packed("set_constant", y);
+  anode_gpu_set_constant_packed_f32(sz2uint(y.shape.flat_len()), c, y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+}
+
+// ---------------------------------------------------------------------------
 // recipes of src/ops.rs on top of the operators
 // ---------------------------------------------------------------------------
 
@@ -467,6 +541,15 @@ inline void batch_normalize(const GPUDeviceConn &conn, float epsilon, const Devi
   BatchMeanOp::apply(WriteCap::Assign, conn, x, mean);
   BatchVarianceOp::apply(WriteCap::Assign, conn, epsilon, x, mean, var);
   BatchNormalizeOp::apply(WriteCap::Assign, conn, x, mean, var, y);
+}
+
+// src/ops.rs:1002-1003: the running statistics follow the batch statistics at `rate`; the running variance tracks
+// the biased variance + epsilon, as the reference's does.
+inline void batch_normalize_update_running(const GPUDeviceConn &conn, float rate, const DeviceArray<float> &mean,
+                                           const DeviceArray<float> &var, DeviceArray<float> &running_mean,
+                                           DeviceArray<float> &running_var) {
+  OnlineAverageOp::apply(conn, rate, mean, running_mean);
+  OnlineAverageOp::apply(conn, rate, var, running_var);
 }
 
 // The adjoint graph of the recipe (src/ops_gpu.rs:4344-4352, 3997-4004, 3787-3795) in the order the sink

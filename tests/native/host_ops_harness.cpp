@@ -231,6 +231,71 @@ int main() {
     check(ok, "positive_clip in place, and its backward in place");
   }
 
+  // ---- running statistics (tests/test_gpu.rs:561-593): 0 -> 0.25 -> 0.4375 at rate 0.25 towards 1 ----
+  {
+    Dev<float> x(std::vector<float>(1024, 1.0f)), y(std::vector<float>(1024, 0.0f));
+    auto xa = array1d(x.p, 1024), ya = array1d(y.p, 1024);
+    OnlineAverageOp::apply(conn, 0.25f, xa, ya);
+    auto h1 = y.host(stream);
+    OnlineAverageOp::apply(conn, 0.25f, xa, ya);
+    auto h2 = y.host(stream);
+    bool ok = true;
+    for (size_t i = 0; i < 1024; ++i) ok = ok && h1[i] == 0.25f && h2[i] == 0.4375f;
+    check(ok, "online_average: 0.25 then 0.4375");
+    OnlineAddOp::apply(conn, 0.5f, xa, ya);
+    auto h3 = y.host(stream);
+    ok = true;
+    for (size_t i = 0; i < 1024; ++i) ok = ok && h3[i] == 0.9375f;
+    check(ok, "online_add: y + 0.5 * x");
+  }
+
+  // ---- batch sum / broadcast / per-sample division / fills (src/ops_gpu.rs:7478-7614, 9575-9605, 1244, 2080) ----
+  {
+    const size_t batch = 10, inner = 37;
+    Dev<float> ones(batch), total(1), spread(batch);
+    auto oa = array1d(ones.p, batch), ta = array1d(total.p, 1), sa = array1d(spread.p, batch);
+    set_constant(conn, 1.0f, oa);
+    BatchSumOp::apply(WriteCap::Assign, conn, oa, ta);
+    check(total.host(stream)[0] == 10.0f, "batch_sum of ten ones == 10 (the sum the reference's sum-join test expects)");
+    BatchSumOp::apply(WriteCap::Accumulate, conn, oa, ta);
+    check(total.host(stream)[0] == 20.0f, "batch_sum Accumulate adds");
+    BatchBroadcastOp::apply(WriteCap::Assign, conn, ta, sa);
+    BatchBroadcastOp::apply(WriteCap::Accumulate, conn, ta, sa);
+    auto hs = spread.host(stream);
+    bool ok = true;
+    for (float v : hs) ok = ok && v == 40.0f;
+    check(ok, "batch broadcast: Assign then Accumulate");
+
+    std::vector<float> hx(inner * batch), hr(batch);
+    uint32_t seed = 99u;
+    for (auto &v : hx) v = frand(seed);
+    for (size_t b = 0; b < batch; ++b) hr[b] = 0.5f + float(b);
+    Dev<float> x(hx), r(hr), y(inner * batch), nz(inner * batch);
+    auto xa = obatch1d(x.p, inner, batch), ra = obatch1d(r.p, 1, batch), ya = obatch1d(y.p, inner, batch);
+    FlatBroadcastRdivOp::apply(WriteCap::Assign, conn, xa, ra, ya);
+    auto hy = y.host(stream);
+    ok = true;
+    for (size_t b = 0; b < batch; ++b)
+      for (size_t a = 0; a < inner; ++a) ok = ok && hy[a + inner * b] == hx[a + inner * b] / hr[b];
+    check(ok, "flat broadcast rdiv: x / r[batch]");
+    bool threw = false;
+    try {
+      FlatBroadcastRdivOp::apply(WriteCap::Accumulate, conn, xa, ra, ya);
+    } catch (const Unimplemented &) {
+      threw = true;
+    }
+    check(threw, "FlatBroadcastRdivOp with WriteCap::Accumulate is unimplemented");
+    hx[3] = 0.0f;
+    hx[5] = -0.0f;
+    Dev<float> x2(hx);
+    auto x2a = obatch1d(x2.p, inner, batch), nza = obatch1d(nz.p, inner, batch);
+    IsNonzeroOp::apply(WriteCap::Assign, conn, x2a, nza);
+    auto hn = nz.host(stream);
+    ok = true;
+    for (size_t i = 0; i < hx.size(); ++i) ok = ok && hn[i] == float(hx[i] != 0.0f);
+    check(ok, "is_nonzero");
+  }
+
   check(anode_gpu_take_last_error() == 0, "no launch error recorded");
   HIP_OK(hipStreamDestroy(stream));
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "ALL PASS", g_checks, g_failed);
