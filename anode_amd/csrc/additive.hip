@@ -494,7 +494,7 @@ ANODE_EXPORT void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, con
   if (dim1 == 0) return;
   const uint32_t waves_per_block = kBlock / kWave;
   uint32_t blocks = (dim1 + waves_per_block - 1) / waves_per_block;
-  const uint32_t cap = uint32_t(device_cu_count()) * 8u;
+  const uint32_t cap = 1u << 24;  // one row per wave; the kernel loops only beyond that
   if (blocks > cap) blocks = cap;
   arg_max_rows_kernel<<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
   note_launch(__func__);

@@ -281,6 +281,28 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_fold_kernel(uint32_t C, ui
   if (lane == 0) op.finalize(c, s0, s1, s2);
 }
 
+// The same for channels with many partials: one workgroup per channel, thread t takes partials t, t+256, ...,
+// then the workgroup sum.
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void chan_reduce_fold_block_kernel(uint32_t C, uint32_t ppc, Op op,
+                                                                        const double *__restrict__ part) {
+  __shared__ double lds[kBlock / kWave];
+  const uint32_t c = blockIdx.x;
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0;
+  const double *p0 = part + size_t(c) * ppc;
+  const double *p1 = p0 + size_t(C) * ppc;
+  const double *p2 = p1 + size_t(C) * ppc;
+  for (uint32_t j = threadIdx.x; j < ppc; j += kBlock) {
+    s0 += p0[j];
+    if (Op::NACC >= 2) s1 += p1[j];
+    if (Op::NACC >= 3) s2 += p2[j];
+  }
+  s0 = block_sum(s0, lds);
+  if (Op::NACC >= 2) s1 = block_sum(s1, lds);
+  if (Op::NACC >= 3) s2 = block_sum(s2, lds);
+  if (threadIdx.x == 0) op.finalize(c, s0, s1, s2);
+}
+
 template <typename Op>
 void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
                         const float *b, CUstream_st *stream, const float *c = nullptr) {
@@ -323,8 +345,12 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
   }
   note_launch(symbol);
   if (pl.ppc > 1) {
-    const uint32_t waves_per_block = kBlock / kWave;
-    chan_reduce_fold_kernel<Op><<<(C + waves_per_block - 1) / waves_per_block, kBlock, 0, s>>>(C, pl.ppc, op, part);
+    if (pl.ppc > 256) {  // few channels, long lists of partials (a scalar sum of a large array)
+      chan_reduce_fold_block_kernel<Op><<<C, kBlock, 0, s>>>(C, pl.ppc, op, part);
+    } else {
+      const uint32_t waves_per_block = kBlock / kWave;
+      chan_reduce_fold_kernel<Op><<<(C + waves_per_block - 1) / waves_per_block, kBlock, 0, s>>>(C, pl.ppc, op, part);
+    }
     note_launch(symbol);
   }
 }

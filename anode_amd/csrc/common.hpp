@@ -138,6 +138,19 @@ __device__ inline T block_sum(T v, T *lds) {
   return total;
 }
 
+// Workgroup maximum, same contract as block_sum.
+__device__ inline float block_max(float v, float *lds) {
+  v = wave_max(v);
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+  __syncthreads();
+  float top = lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, lds[w]);
+  __syncthreads();
+  return top;
+}
+
 #endif  // __HIPCC__
 
 // ---------------------------------------------------------------------------

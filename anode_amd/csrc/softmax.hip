@@ -1,8 +1,10 @@
 // Softmax with the categorical negative log-likelihood gather and its backward.
 //
 // Row form  [K classes (fastest), R rows]: the reduced axis is contiguous.
-//   K <= 64     : a row lives in a power-of-two group of lanes, several rows per wave;
+//   K <= 32     : one thread per row; a workgroup's 256 rows are staged through LDS with coalesced accesses;
+//   K <= 64     : a row lives in a group of 64 lanes;
 //   K <= 2048   : one wave per row, the row held in registers (lane l owns k = l, l+64, ...);
+//   K <= 16384  : one workgroup per row, the row held in registers;
 //   larger K    : one workgroup per row, online max/sum pass then a normalising pass.
 // N-d form  [P pixels (fastest), C classes, N]: the reduced axis has stride P.
 //   One thread owns 4 consecutive pixels (16-byte accesses, coalesced across the
@@ -45,6 +47,89 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
     const float z = valid ? expf(v - m) : 0.0f;
     const float s = group_sum(z, int(G));
     if (valid) y[idx] = z / s;
+  }
+}
+
+// K <= KMAX <= 32: one thread per row.  A workgroup takes 256 consecutive rows, which are 256*K contiguous floats:
+// they are copied to LDS with full-width coalesced loads (row pitch K|1, so that threads reading their own row hit
+// distinct banks), each thread normalises its row in registers, and the tile goes back the same way.  No cross-lane
+// traffic at all, which is what bounds the lane-group kernel below for short rows.
+template <int KMAX>
+__global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, FastDiv div_k, int vec,
+                                                                 const float *__restrict__ x,
+                                                                 float *__restrict__ y) {
+  extern __shared__ float tile[];  // kBlock * (K|1) floats
+  const uint32_t pitch = K | 1u;
+  for (uint64_t r0 = uint64_t(blockIdx.x) * kBlock; r0 < R; r0 += uint64_t(gridDim.x) * kBlock) {
+    const uint32_t rows = (R - r0 < uint64_t(kBlock)) ? uint32_t(R - r0) : uint32_t(kBlock);
+    const uint32_t n = rows * K;
+    const float *xt = x + r0 * K;
+    float *yt = y + r0 * K;
+    const uint32_t n4 = vec ? n / 4u : 0u;  // the tile starts 1024*K bytes into an aligned array: 16-byte aligned
+    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
+      const f32x4 v = reinterpret_cast<const f32x4 *>(xt)[g];
+      uint32_t q, c;
+      div_k.divmod(g * 4u, q, c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        tile[q * pitch + c] = v[j];
+        if (++c == K) {
+          c = 0;
+          ++q;
+        }
+      }
+    }
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
+      uint32_t q, c;
+      div_k.divmod(e, q, c);
+      tile[q * pitch + c] = xt[e];
+    }
+    __syncthreads();
+    if (threadIdx.x < rows) {
+      float *row = tile + threadIdx.x * pitch;
+      float v[KMAX];
+      float m = kNegInf;
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) {
+        if (uint32_t(k) < K) {
+          v[k] = row[k];
+          m = fmaxf(m, v[k]);
+        }
+      }
+      float sum = 0.0f;
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) {
+        if (uint32_t(k) < K) {
+          v[k] = expf(v[k] - m);
+          sum += v[k];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) {
+        if (uint32_t(k) < K) row[k] = v[k] / sum;
+      }
+    }
+    __syncthreads();
+    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
+      uint32_t q, c;
+      div_k.divmod(g * 4u, q, c);
+      f32x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[j] = tile[q * pitch + c];
+        if (++c == K) {
+          c = 0;
+          ++q;
+        }
+      }
+      reinterpret_cast<f32x4 *>(yt)[g] = v;
+    }
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
+      uint32_t q, c;
+      div_k.divmod(e, q, c);
+      yt[e] = tile[q * pitch + c];
+    }
+    __syncthreads();  // the tile is overwritten by the next pass
   }
 }
 
@@ -94,7 +179,41 @@ __device__ inline void online_merge(float &m, float &s, float m2, float s2) {
   m = mm;
 }
 
-// any K: one workgroup per row
+// 2048 < K <= 256 * VPT: one workgroup per row, the row in registers (VPT values per thread), so x is read once.
+template <int VPT>
+__global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K, uint32_t R,
+                                                                      const float *__restrict__ x,
+                                                                      float *__restrict__ y) {
+  __shared__ float lds[kBlock / kWave];
+  for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
+    const float *xr = x + size_t(r) * K;
+    float *yr = y + size_t(r) * K;
+    float v[VPT];
+    float m = kNegInf;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
+      v[i] = (k < K) ? xr[k] : kNegInf;
+      m = fmaxf(m, v[i]);
+    }
+    m = block_max(m, lds);
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
+      v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
+      s += v[i];
+    }
+    s = block_sum(s, lds);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
+      if (k < K) yr[k] = v[i] / s;
+    }
+  }
+}
+
+// any K: one workgroup per row, the row streamed twice
 __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, uint32_t R,
                                                                    const float *__restrict__ x,
                                                                    float *__restrict__ y) {
@@ -138,9 +257,26 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   (void)checked_len(K, R, 1, symbol);
   if (K == 0 || R == 0) return;
   hipStream_t s = as_stream(stream);
-  const uint32_t max_blocks = uint32_t(device_cu_count()) * 8u;
+  // one row (or group of rows) per wave / workgroup and a grid that covers all of them: the loop in the kernels
+  // only runs again when the row count exceeds the grid limit
+  const uint32_t max_blocks = 1u << 24;
   constexpr uint32_t kWavesPerBlock = kBlock / kWave;
-  if (K <= 64) {
+  if (K <= 32) {
+    uint32_t blocks = (R + kBlock - 1) / kBlock;
+    if (blocks > max_blocks) blocks = max_blocks;
+    const size_t lds_bytes = size_t(kBlock) * (K | 1u) * sizeof(float);
+    const FastDiv div_k(K);
+    const int vec = (aligned16(x) && aligned16(y)) ? 1 : 0;
+    if (K <= 4) {
+      softmax_row_lds_kernel<4><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+    } else if (K <= 8) {
+      softmax_row_lds_kernel<8><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+    } else if (K <= 16) {
+      softmax_row_lds_kernel<16><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+    } else {
+      softmax_row_lds_kernel<32><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+    }
+  } else if (K <= 64) {
     uint32_t log2g = 0;
     while ((1u << log2g) < K) ++log2g;
     const uint32_t rows_per_block = kWavesPerBlock * (64u >> log2g);
@@ -162,8 +298,16 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       softmax_row_wave_kernel<32><<<blocks, kBlock, 0, s>>>(K, R, x, y);
     }
   } else {
-    uint32_t blocks = R < max_blocks ? R : max_blocks;
-    softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    const uint32_t blocks = R < max_blocks ? R : max_blocks;
+    if (K <= 4096) {
+      softmax_row_blockreg_kernel<16><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else if (K <= 8192) {
+      softmax_row_blockreg_kernel<32><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else if (K <= 16384) {
+      softmax_row_blockreg_kernel<64><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    } else {
+      softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    }
   }
   note_launch(symbol);
 }

@@ -38,6 +38,8 @@ def parse_args():
     ap.add_argument("--stream-probe", action="store_true",
                     help="instead of the benchmark: time the library's plain copy and a read-only reduction on cold "
                          "822 MB arrays under the launch-geometry and cache-policy knobs, one JSON line")
+    ap.add_argument("--all-symbols", action="store_true",
+                    help="instead of the benchmark: every entry point once at a bandwidth-sized shape, one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="add one plain copy of a known size to the step (scale for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
@@ -212,6 +214,124 @@ def stream_probe(torch, gpu):
     return out
 
 
+def all_symbols(torch, gpu):
+    """Every entry point of the reference ABI (and the additive ones) once, at a bandwidth-sized shape: median time
+    of 7 launches made in rotation with the others (so each launch meets a cold cache), algorithmic bytes / time."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    E = lambda n, dt=torch.float32: torch.empty(n, device="cuda", dtype=dt)  # noqa: E731
+    Rn = lambda n: torch.randn(n, device="cuda", generator=g)                # noqa: E731
+    L = []
+
+    def add(symbol, shape, args, nbytes):
+        L.append((symbol, shape, args, nbytes))
+
+    # batch-norm family on [256,64,112,112]
+    S, C, N = 112 * 112, 64, 256
+    n = S * C * N
+    d = (S, C, N)
+    x, dy, y, dx = Rn(n), Rn(n), E(n), Rn(n)
+    m, v, dm, dv = Rn(C), torch.rand(C, device="cuda", generator=g) + 0.5, Rn(C), Rn(C)
+    sh = "[256,64,112,112]"
+    add("anode_gpu_batch_mean_3d1_packed_f32", sh, (*d, x, E(C)), 4 * n)
+    add("anode_gpu_batch_var_3d1_packed_f32", sh, (*d, 1e-5, x, m, E(C)), 4 * n)
+    add("anode_gpu_batch_norm_3d1_packed_f32", sh, (*d, x, m, v, y), 8 * n)
+    add("anode_gpu_batch_norm_bwd_3d1_packed_f32", sh, (*d, dy, v, y), 8 * n)
+    add("anode_gpu_batch_norm_bwd_3d1_packed_accumulate_f32", sh, (*d, dy, v, dx), 12 * n)
+    add("anode_gpu_batch_norm_bwd_mean_3d1_packed_f32", sh, (*d, dy, v, E(C)), 4 * n)
+    add("anode_gpu_batch_norm_bwd_mean_3d1_packed_accumulate_f32", sh, (*d, dy, v, dm), 4 * n)
+    add("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", sh, (*d, dy, x, m, v, E(C)), 8 * n)
+    add("anode_gpu_batch_norm_bwd_var_3d1_packed_accumulate_f32", sh, (*d, dy, x, m, v, dv), 8 * n)
+    add("anode_gpu_batch_norm_bwd_var_v2_3d1_packed_f32", sh, (*d, dy, x, v, E(C)), 8 * n)
+    add("anode_gpu_batch_norm_bwd_var_v2_3d1_packed_accumulate_f32", sh, (*d, dy, x, v, dv), 8 * n)
+    add("anode_gpu_batch_var_bwd_3d1_packed_f32", sh, (*d, dv, x, m, y), 8 * n)
+    add("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", sh, (*d, dv, x, m, dx), 12 * n)
+    add("anode_gpu_batch_var_bwd_mean_3d1_packed_f32", sh, (*d, dv, x, m, E(C)), 4 * n)
+    add("anode_gpu_batch_var_bwd_mean_3d1_packed_accumulate_f32", sh, (*d, dv, x, m, dm), 4 * n)
+    add("anode_gpu_batch_mean_bwd_3d1_packed_f32", sh, (*d, dm, y), 4 * n)
+    add("anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32", sh, (*d, dm, dx), 8 * n)
+    # additive batch-norm entry points on the same arrays
+    add("anode_gpu_batch_mean_var_3d1_packed_f32", sh, (*d, 1e-5, x, E(C), E(C)), 4 * n)
+    add("anode_gpu_batch_norm_positive_clip_3d1_packed_f32", sh, (*d, x, m, v, y), 8 * n)
+    add("anode_gpu_batch_norm_affine_3d1_packed_f32", sh, (*d, x, m, v, dm, dv, y), 8 * n)
+    add("anode_gpu_batch_norm_bwd_reduce_3d1_packed_f32", sh, (*d, dy, x, m, v, None, E(C), E(C)), 8 * n)
+    add("anode_gpu_batch_norm_bwd_apply_3d1_packed_f32", sh, (*d, dy, x, m, v, dm, dv, None, y), 12 * n)
+    add("anode_gpu_bcast_flat_mult_add_I1b_I2abc_Oabc_packed_f32", sh, (*d, dm, x, dv, y), 8 * n)
+
+    # flat maps and the join on the same 822 MB arrays
+    fl = f"[{n}]"
+    for name in ("copy", "modulus", "square", "sqrt", "positive_clip", "logistic", "unit_step", "normal_cdf", "tanh",
+                 "rcosh2"):
+        add(f"anode_gpu_{name}_flat_map_f32", fl, (n, x, y), 8 * n)
+    add("anode_gpu_leaky_relu_flat_map_f32", fl, (n, 0.1, x, y), 8 * n)
+    add("anode_gpu_positive_clip_flat_map_bwd_f32", fl, (n, dy, x, y), 12 * n)
+    add("anode_gpu_logistic_flat_map_bwd_f32", fl, (n, dy, x, y), 12 * n)
+    add("anode_gpu_leaky_relu_flat_map_bwd_f32", fl, (n, 0.1, dy, x, y), 12 * n)
+    add("anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32", fl, (n, dy, x, y), 12 * n)
+    add("anode_gpu_add_packed_f32", fl, (n, x, dx), 12 * n)
+    add("anode_gpu_set_constant_packed_f32", fl, (n, 0.0, y), 4 * n)
+    add("anode_gpu_sum_packed_deterministic_f32", fl, (n, x, E(1)), 4 * n)
+
+    # casts on [256,3,224,224]
+    nq = 256 * 3 * 224 * 224
+    q = torch.randint(0, 256, (nq,), device="cuda", dtype=torch.uint8, generator=g)
+    add("anode_gpu_dequantize_u8_packed_f32", "[256,3,224,224]", (nq, 0.0, 1.0, q, y), 5 * nq)
+    add("anode_gpu_upcast_u8_packed_u32", "[256,3,224,224]", (nq, q, E(nq, torch.int32)), 5 * nq)
+    add("anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32", "[256,3,224,224]",
+        (224 * 224, 3, 256, Rn(3), Rn(3), q, y), 5 * nq)
+    add("anode_gpu_quantize_u8_packed_f32", "[256,3,224,224]", (nq, -4.0, 4.0, x, E(nq, torch.uint8)), 5 * nq)
+
+    # row softmax / NLL: K = 10, 1000, 4096
+    for K, R in ((10, 4 << 20), (1000, 65536), (4096, 16384)):
+        lab = torch.randint(0, K, (R,), device="cuda", dtype=torch.int32, generator=g)
+        rs = f"[{R},{K}]"
+        add("anode_gpu_softmax_packed_block_f32", rs, (K, R, x, y), 8 * K * R)
+        add("anode_gpu_softmax_packed_deterministic_f32", rs, (K, R, x, y), 8 * K * R)
+        if K == 1000:
+            add("anode_gpu_softmax_cat_nll_packed_f32", rs, (K, R, x, lab, E(R)), 12 * R)
+            add("anode_gpu_softmax_cat_nll_bwd_packed_f32", rs, (K, R, dy, x, lab, y), 8 * K * R + 8 * R)
+            add("anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32", rs, (K, R, dy, x, lab, dx), 12 * K * R + 8 * R)
+            add("anode_gpu_arg_max_packed_u32", rs, (K, R, x, E(R, torch.int32)), 4 * K * R + 4 * R)
+
+    # channel-axis softmax / NLL / one-hot / F1 on [8,19,512,1024]
+    P, Cc, Nn = 512 * 1024, 19, 8
+    ns = P * Cc * Nn
+    lab = torch.randint(0, Cc, (P * Nn,), device="cuda", dtype=torch.int32, generator=g)
+    ss = "[8,19,512,1024]"
+    add("anode_gpu_softmax_nd_packed_f32", ss, (P, Cc, Nn, x, y), 8 * ns)
+    add("anode_gpu_softmax_nd_cat_nll_packed_f32", ss, (P, Cc, Nn, x, lab, E(P * Nn)), 12 * P * Nn)
+    add("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", ss, (P, Cc, Nn, dy, x, lab, y), 8 * ns + 8 * P * Nn)
+    add("anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32", ss, (P, Cc, Nn, dy, x, lab, dx), 12 * ns + 8 * P * Nn)
+    add("anode_gpu_softmax_nd_cat_nll_fused_packed_f32", ss, (P, Cc, Nn, x, lab, y, E(P * Nn)), 8 * ns + 8 * P * Nn)
+    add("anode_gpu_discrete_one_hot_3d1_packed_f32", ss, (P, Cc, Nn, lab, y), 4 * P * Nn + 4 * ns)
+    t01 = (torch.rand(ns, device="cuda", generator=g) < 0.3).float()
+    add("anode_gpu_smooth_negative_f1_loss_3d1_packed_f32", ss, (P, Cc, Nn, 1e-3, x, t01, E(Cc * Nn)), 8 * ns)
+    add("anode_gpu_smooth_negative_f1_loss_3d1_bwd_packed_f32", ss, (P, Cc, Nn, 1e-3, Rn(Cc * Nn), x, t01, y), 12 * ns)
+
+    for sym, _, args, _ in L:
+        gpu.call(sym, *args)
+    torch.cuda.synchronize()
+    times = [[] for _ in L]
+    for _ in range(7):
+        evs = []
+        for sym, _, args, _ in L:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            gpu.call(sym, *args)
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(evs):
+            times[i].append(a.elapsed_time(b) * 1e-3)
+    assert gpu.take_last_error() == 0
+    rows = []
+    for (sym, shape, _, nbytes), t in zip(L, times):
+        t = sorted(t)[len(t) // 2]
+        rows.append({"symbol": sym.replace("anode_gpu_", ""), "shape": shape, "us": round(t * 1e6, 1),
+                     "gbps": round(nbytes / t / 1e9, 1), "pct_of_peak": round(100 * nbytes / t / 1e9 / HBM_PEAK_GBPS, 1)})
+    return rows
+
+
 def small_shape_latency(torch, gpu, groups, passes=100):
     """Launch-bound shapes (config 0, config 3a): time per pass over `passes` back-to-back passes, launched one entry
     point at a time and as one captured HIP graph replayed.  Separates launch latency from bandwidth."""
@@ -378,6 +498,9 @@ def main():
     torch.cuda.set_device(0)
     if args.stream_probe:
         print(json.dumps({"stream_probe": stream_probe(torch, gpu)}), flush=True)
+        return
+    if args.all_symbols:
+        print(json.dumps({"all_symbols": all_symbols(torch, gpu), "peak_gbps": HBM_PEAK_GBPS}), flush=True)
         return
     only = set(filter(None, args.only.split(",")))
     launches, fused = build_workload(torch, only, args.copy_calibration)
