@@ -573,6 +573,8 @@ void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x
     softmax_nd_reg_kernel<8, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 16) {
     softmax_nd_reg_kernel<16, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+  } else if (C <= 20) {  // 19 / 20 classes are common label sets; four registers per class saved buy a wave of occupancy
+    softmax_nd_reg_kernel<20, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 24) {
     softmax_nd_reg_kernel<24, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else {

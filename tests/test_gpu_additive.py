@@ -206,8 +206,9 @@ def test_ref_online_average_quarter_steps(oracle):
 
 def test_arg_max_rows(oracle):
     g = np.random.default_rng(3)
-    for K, R in [(10, 32), (1000, 256), (1, 5), (64, 7), (65, 3), (5000, 2)]:
-        x = g.standard_normal(K * R).astype(F32)
+    for K, R in [(10, 32), (1000, 256), (1, 5), (64, 7), (65, 3), (5000, 2), (1001, 33), (8, 1000), (4096, 9)]:
+        # a coarse grid of values: ties within a lane's group of four, across lanes and across loop passes
+        x = (g.integers(-3, 4, K * R) * 0.5).astype(F32) if K in (8, 1001, 4096) else g.standard_normal(K * R).astype(F32)
         xr = x.reshape(R, K)
         if R > 3 and K > 4:
             xr[0, :] = 1.0                       # all equal: first index
@@ -215,6 +216,7 @@ def test_arg_max_rows(oracle):
             xr[2, 0] = np.nan
             xr[2, 3] = np.nan                    # NaN never wins
             xr[3, K - 1] = xr[3, K - 2] = 9.0    # tie: the first of the two
-        out = empty(R, dtype=torch.int32)
-        call("anode_gpu_arg_max_packed_u32", K, R, dev(x), out)
-        assert_bit_exact(host(out).view(np.uint32), oracle.arg_max_rows(K, R, x), f"arg_max K={K}")
+        for offset in (0, 1):  # aligned rows take the 16-byte path when K is a multiple of 4
+            out = empty(R, dtype=torch.int32)
+            call("anode_gpu_arg_max_packed_u32", K, R, dev(x, offset), out)
+            assert_bit_exact(host(out).view(np.uint32), oracle.arg_max_rows(K, R, x), f"arg_max K={K} offset={offset}")
