@@ -133,11 +133,14 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
   }
 }
 
-// 64 < K <= 64 * VPL: one wave per row, VPL values per lane.
-template <int VPL>
+// 64 < K <= 64 * VPL: one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
+// of 4, aligned arrays) and a lane owns groups of four consecutive classes; otherwise lane l owns k = l, l+64, ...
+template <int VPL, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
                                                                   const float *__restrict__ x,
                                                                   float *__restrict__ y) {
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int NG = VPL / W;  // groups per lane
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t n_waves = gridDim.x * (kBlock / kWave);
@@ -147,24 +150,41 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
     float v[VPL];
     float m = kNegInf;
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const uint32_t k = lane + uint32_t(i) * kWave;
-      v[i] = (k < K) ? xr[k] : kNegInf;
-      m = fmaxf(m, v[i]);
+    for (int i = 0; i < NG; ++i) {
+      const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
+      if (VEC) {
+        const f32x4 t = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k))
+                                : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[i * W + j] = t[j];
+          m = fmaxf(m, t[j]);
+        }
+      } else {
+        v[i] = (k < K) ? xr[k] : kNegInf;
+        m = fmaxf(m, v[i]);
+      }
     }
     m = wave_max(m);
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
-      const uint32_t k = lane + uint32_t(i) * kWave;
+      const uint32_t k = (lane + uint32_t(i / W) * kWave) * uint32_t(W) + uint32_t(i % W);
       v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
       s += v[i];
     }
     s = wave_sum(s);
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const uint32_t k = lane + uint32_t(i) * kWave;
-      if (k < K) yr[k] = v[i] / s;
+    for (int i = 0; i < NG; ++i) {
+      const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
+      if (k < K) {
+        if (VEC) {
+          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k),
+                           f32x4{v[i * W] / s, v[i * W + 1] / s, v[i * W + 2] / s, v[i * W + 3] / s});
+        } else {
+          yr[k] = v[i] / s;
+        }
+      }
     }
   }
 }
@@ -180,10 +200,13 @@ __device__ inline void online_merge(float &m, float &s, float m2, float s2) {
 }
 
 // 2048 < K <= 256 * VPT: one workgroup per row, the row in registers (VPT values per thread), so x is read once.
-template <int VPT>
+// VEC as in the wave kernel.
+template <int VPT, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K, uint32_t R,
                                                                       const float *__restrict__ x,
                                                                       float *__restrict__ y) {
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int NG = VPT / W;
   __shared__ float lds[kBlock / kWave];
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
@@ -191,24 +214,41 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
     float v[VPT];
     float m = kNegInf;
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
-      v[i] = (k < K) ? xr[k] : kNegInf;
-      m = fmaxf(m, v[i]);
+    for (int i = 0; i < NG; ++i) {
+      const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
+      if (VEC) {
+        const f32x4 t = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k))
+                                : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[i * W + j] = t[j];
+          m = fmaxf(m, t[j]);
+        }
+      } else {
+        v[i] = (k < K) ? xr[k] : kNegInf;
+        m = fmaxf(m, v[i]);
+      }
     }
     m = block_max(m, lds);
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
+      const uint32_t k = (threadIdx.x + uint32_t(i / W) * kBlock) * uint32_t(W) + uint32_t(i % W);
       v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
       s += v[i];
     }
     s = block_sum(s, lds);
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const uint32_t k = threadIdx.x + uint32_t(i) * kBlock;
-      if (k < K) yr[k] = v[i] / s;
+    for (int i = 0; i < NG; ++i) {
+      const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
+      if (k < K) {
+        if (VEC) {
+          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k),
+                           f32x4{v[i * W] / s, v[i * W + 1] / s, v[i * W + 2] / s, v[i * W + 3] / s});
+        } else {
+          yr[k] = v[i] / s;
+        }
+      }
     }
   }
 }
@@ -261,6 +301,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   // only runs again when the row count exceeds the grid limit
   const uint32_t max_blocks = 1u << 24;
   constexpr uint32_t kWavesPerBlock = kBlock / kWave;
+  const int nt = stream_policy(size_t(K) * R * sizeof(float), tuning().nontemporal);  // logits in, probabilities out: both streamed
   if (K <= 32) {
     uint32_t blocks = (R + kBlock - 1) / kBlock;
     if (blocks > max_blocks) blocks = max_blocks;
@@ -286,28 +327,50 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   } else if (K <= 2048) {
     uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > max_blocks) blocks = max_blocks;
-    if (K <= 128) {
-      softmax_row_wave_kernel<2><<<blocks, kBlock, 0, s>>>(K, R, x, y);
-    } else if (K <= 256) {
-      softmax_row_wave_kernel<4><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
+#define ANODE_ROW_WAVE(VPL)                                                              \
+  do {                                                                                   \
+    if (vec && nt) {                                                                     \
+      softmax_row_wave_kernel<VPL, true, kNtLoad | kNtStore><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+    } else if (vec) {                                                                    \
+      softmax_row_wave_kernel<VPL, true, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);       \
+    } else {                                                                             \
+      softmax_row_wave_kernel<VPL, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);      \
+    }                                                                                    \
+  } while (0)
+    if (K <= 256) {
+      ANODE_ROW_WAVE(4);
     } else if (K <= 512) {
-      softmax_row_wave_kernel<8><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_WAVE(8);
     } else if (K <= 1024) {
-      softmax_row_wave_kernel<16><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_WAVE(16);
     } else {
-      softmax_row_wave_kernel<32><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_WAVE(32);
     }
+#undef ANODE_ROW_WAVE
   } else {
     const uint32_t blocks = R < max_blocks ? R : max_blocks;
+    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
+#define ANODE_ROW_BLOCKREG(VPT)                                                          \
+  do {                                                                                   \
+    if (vec && nt) {                                                                     \
+      softmax_row_blockreg_kernel<VPT, true, kNtLoad | kNtStore><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+    } else if (vec) {                                                                    \
+      softmax_row_blockreg_kernel<VPT, true, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);   \
+    } else {                                                                             \
+      softmax_row_blockreg_kernel<VPT, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);  \
+    }                                                                                    \
+  } while (0)
     if (K <= 4096) {
-      softmax_row_blockreg_kernel<16><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_BLOCKREG(16);
     } else if (K <= 8192) {
-      softmax_row_blockreg_kernel<32><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_BLOCKREG(32);
     } else if (K <= 16384) {
-      softmax_row_blockreg_kernel<64><<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      ANODE_ROW_BLOCKREG(64);
     } else {
       softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y);
     }
+#undef ANODE_ROW_BLOCKREG
   }
   note_launch(symbol);
 }
