@@ -648,6 +648,24 @@ def main():
         "per_symbol": per_symbol,
     }
     if not only:
+        # the same step captured once as a HIP graph and replayed: what the launch gaps cost (reported beside `value`,
+        # which stays the plainly launched figure)
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            run_step()  # the reductions' scratch for this stream exists before capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run_step()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        g_s = (time.perf_counter() - t0) / args.steps
+        out["graph_replay"] = {"ms_per_step": round(g_s * 1e3, 4), "gbps": round(step_bytes / g_s / 1e9, 1),
+                               "pct_of_hbm_peak": round(100 * step_bytes / g_s / 1e9 / HBM_PEAK_GBPS, 2)}
         out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
