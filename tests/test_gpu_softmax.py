@@ -130,7 +130,9 @@ def test_softmax_cat_nll_and_bwd_rows(oracle, K, R):
 # ---- n-d form ----
 
 ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100, 1, 3), (36, 4, 2), (40, 8, 3),
-             (28, 16, 2), (12, 24, 2), (16, 32, 2), (8, 33, 2), (8, 64, 3), (6, 100, 2), (4, 130, 2), (7, 40, 3)]
+             (28, 16, 2), (12, 24, 2), (16, 32, 2), (8, 33, 2), (8, 64, 3), (6, 100, 2), (4, 130, 2), (7, 40, 3),
+             # several waves of pixel groups with a ragged last wave, few and many classes
+             (1300, 19, 3), (516, 32, 5), (1028, 2, 3)]
 
 
 @pytest.mark.parametrize("P,C,N", ND_SHAPES)
