@@ -216,7 +216,7 @@ def stream_probe(torch, gpu):
 
 def all_symbols(torch, gpu):
     """Every entry point of the reference ABI (and the additive ones) once, at a bandwidth-sized shape: median time
-    of 7 launches made in rotation with the others (so each launch meets a cold cache), algorithmic bytes / time."""
+    of 50 launches made in rotation with the others (so each launch meets a cold cache), algorithmic bytes / time."""
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
     E = lambda n, dt=torch.float32: torch.empty(n, device="cuda", dtype=dt)  # noqa: E731
@@ -312,7 +312,7 @@ def all_symbols(torch, gpu):
         gpu.call(sym, *args)
     torch.cuda.synchronize()
     times = [[] for _ in L]
-    for _ in range(7):
+    for _ in range(50):
         evs = []
         for sym, _, args, _ in L:
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -325,9 +325,10 @@ def all_symbols(torch, gpu):
             times[i].append(a.elapsed_time(b) * 1e-3)
     assert gpu.take_last_error() == 0
     rows = []
-    for (sym, shape, _, nbytes), t in zip(L, times):
-        t = sorted(t)[len(t) // 2]
+    for (sym, shape, _, nbytes), ts in zip(L, times):
+        t = sorted(ts)[len(ts) // 2]
         rows.append({"symbol": sym.replace("anode_gpu_", ""), "shape": shape, "us": round(t * 1e6, 1),
+                     "min_us": round(min(ts) * 1e6, 1),
                      "gbps": round(nbytes / t / 1e9, 1), "pct_of_peak": round(100 * nbytes / t / 1e9 / HBM_PEAK_GBPS, 1)})
     return rows
 
@@ -525,7 +526,7 @@ def main():
 
     # untimed calibration pass: per-launch HIP-event durations for the breakdown
     per_launch = [[] for _ in launches]
-    for _ in range(3):
+    for _ in range(10):
         evs = []
         for l in launches:
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -575,7 +576,8 @@ def main():
     breakdown = {k: {"gbps": round(b / s / 1e9, 1), "pct_of_peak": round(100 * b / s / 1e9 / HBM_PEAK_GBPS, 1),
                      "us": round(s * 1e6, 1), "gelem_per_s": round(e / s / 1e9, 2)} for k, (b, s, e) in groups.items()}
     per_symbol = [{"group": l.group, "symbol": l.symbol.replace("anode_gpu_", ""), "us": round(t * 1e6, 1),
-                   "gbps": round(l.alg_bytes / t / 1e9, 1)} for l, t in zip(launches, med)]
+                   "min_us": round(min(ts) * 1e6, 1), "gbps": round(l.alg_bytes / t / 1e9, 1)}
+                  for l, t, ts in zip(launches, med, per_launch)]
 
     # the additive (fused) entry points on the same data: time per group over the fused byte model, and the
     # time of the reference-ABI launches that do the same work
