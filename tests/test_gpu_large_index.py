@@ -95,3 +95,77 @@ def test_softmax_nd_beyond_2_31(big):
     sums = pv.sum(dim=1)
     assert bool(((sums - 1).abs() < 1e-5).all())
     del p, sums
+
+
+# ---- close to the largest array the 32-bit counts of the ABI can describe: 2^32 - 3 elements (17 GB) ----
+
+N_MAX = (1 << 32) - 3
+
+
+@pytest.fixture(scope="module")
+def huge():
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    x = torch.empty(N_MAX + 4, device="cuda")
+    x.normal_(generator=g)
+    yield x
+    del x
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("offset", [0, 1])
+def test_flat_map_and_accumulate_close_to_2_32(huge, offset):
+    x = huge[offset:offset + N_MAX]
+    y = torch.full((N_MAX + 4,), float("nan"), device="cuda")
+    call("anode_gpu_positive_clip_flat_map_f32", N_MAX, x, y[offset:offset + N_MAX])
+    torch.cuda.synchronize()
+    want = torch.relu(x)
+    assert torch.equal(y[offset:offset + N_MAX], want)
+    assert bool(torch.isnan(y[offset + N_MAX:]).all()) and bool(torch.isnan(y[:offset]).all())
+    call("anode_gpu_add_packed_f32", N_MAX, x, y[offset:offset + N_MAX])   # y = relu(x) + x, applied exactly once
+    torch.cuda.synchronize()
+    want += x
+    assert torch.equal(y[offset:offset + N_MAX], want)
+    del y, want
+
+
+def test_batch_norm_pieces_close_to_2_32(huge):
+    S, C, N = 1 << 20, 3, 1365           # 4 293 918 720 elements
+    n = S * C * N
+    assert n < (1 << 32) and n > N_MAX - (1 << 21)
+    x = huge[:n]
+    mean, var = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, x, mean)
+    call("anode_gpu_batch_var_3d1_packed_f32", S, C, N, 1e-5, x, mean, var)
+    y = torch.empty(n, device="cuda")
+    call("anode_gpu_batch_norm_3d1_packed_f32", S, C, N, x, mean, var, y)
+    torch.cuda.synchronize()
+    xv, yv = x.view(N, C, S), y.view(N, C, S)
+    for c in range(C):
+        m = xv[:, c, :].mean(dtype=torch.float64).item()
+        v = xv[:, c, :].var(unbiased=False).item() + 1e-5
+        assert abs(float(mean[c]) - m) <= 1e-5 * abs(m) + 1e-7
+        assert abs(float(var[c]) - v) <= 2e-5 * v        # torch's own fp32 variance is the looser side here
+        ym = yv[:, c, :].mean(dtype=torch.float64).item()
+        yq = (yv[:, c, :].double() ** 2).mean().item() if c == C - 1 else None
+        assert abs(ym) < 1e-4
+        if yq is not None:                                 # the last channel ends at the last element of the array
+            assert abs(yq - (1 - 1e-5 / v)) < 1e-4
+    del y
+
+
+def test_softmax_nd_close_to_2_32(huge):
+    P, C, N = 1 << 16, 19, 3449          # 4 294 639 616 elements
+    n = P * C * N
+    assert n < (1 << 32)
+    x = huge[:n]
+    p = torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_packed_f32", P, C, N, x, p)
+    torch.cuda.synchronize()
+    pv = p.view(N, C, P)
+    for i in (0, N // 2, N - 1):
+        ref = torch.softmax(x.view(N, C, P)[i].double(), dim=0)
+        assert bool(((pv[i].double() - ref).abs() <= 1e-5 * ref).all())
+    sums = pv.sum(dim=1)
+    assert bool(((sums - 1).abs() < 1e-5).all())
+    del p, sums
