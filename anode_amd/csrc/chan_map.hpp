@@ -48,7 +48,10 @@ __device__ inline float chan_map_apply(const Op &op, const P &p, float x, float 
   }
 }
 
-template <typename V, int NIN, bool ACC, int UNROLL, int NT, typename Op>
+// PAIR selects how a group that crosses a channel boundary gets its second parameter set: fetched up front beside
+// the first (channels of a few dozen elements, where a quarter of the groups cross), or on demand while walking
+// the group (long channels, where almost none does and the extra fetch and selects only cost issue slots).
+template <typename V, int NIN, bool ACC, int UNROLL, int NT, bool PAIR, typename Op>
 __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
                                                           FastDiv div_c, Op op, const float *a_,
                                                           const float *b_, const float *c_, float *out_) {
@@ -79,20 +82,46 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
         uint32_t q, s;
         div_s.divmod(uint32_t(g) * uint32_t(L), q, s);
         uint32_t c = q - div_c.div(q) * C;
-        typename Op::Param p = op.load(c);
         V r;
+        if (PAIR) {  // the host guarantees S >= L here
+          // A group spans at most two channels.  Both parameter sets are fetched up front, next to the element
+          // loads, so that a group that crosses a channel boundary does not wait for a second, dependent fetch
+          // (with S = 49 a quarter of the groups cross).
+          const uint32_t room = S - s;  // elements of the group that still belong to channel c
+          const typename Op::Param p0 = op.load(c);
+          const uint32_t c1 = (c + 1 == C) ? 0 : c + 1;
+          const typename Op::Param p1 = (room < uint32_t(L)) ? op.load(c1) : p0;
 #pragma unroll
-        for (int k = 0; k < L; ++k) {
-          const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
-          const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
-          const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
-          const float v = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? lane_get<V>(vo[u], k) : 0.0f);
-          lane_set<V>(r, k, v);
-          if (k + 1 < L) {
-            if (++s == S) {
-              s = 0;
-              c = (c + 1 == C) ? 0 : c + 1;
-              p = op.load(c);
+          for (int k = 0; k < L; ++k) {
+            const bool first = uint32_t(k) < room;
+            const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
+            const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
+            const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
+            const float old = ACC ? lane_get<V>(vo[u], k) : 0.0f;
+            if (L == 1) {
+              lane_set<V>(r, k, chan_map_apply<NIN, ACC>(op, p0, x, y, z, s, old));
+            } else {
+              const typename Op::Param pk = first ? p0 : p1;
+              const uint32_t sk = first ? s + uint32_t(k) : uint32_t(k) - room;
+              lane_set<V>(r, k, chan_map_apply<NIN, ACC>(op, pk, x, y, z, sk, old));
+            }
+          }
+        } else {
+          // channels shorter than a group: walk (s, c) element by element
+          typename Op::Param p = op.load(c);
+#pragma unroll
+          for (int k = 0; k < L; ++k) {
+            const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
+            const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
+            const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
+            const float v = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? lane_get<V>(vo[u], k) : 0.0f);
+            lane_set<V>(r, k, v);
+            if (k + 1 < L) {
+              if (++s == S) {
+                s = 0;
+                c = (c + 1 == C) ? 0 : c + 1;
+                p = op.load(c);
+              }
             }
           }
         }
@@ -127,15 +156,22 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
-    if (nt) {
-      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, Op>
+    const bool pair = S >= 4 && S < 4096;
+    if (nt && pair) {
+      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, true, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+    } else if (nt) {
+      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, false, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+    } else if (pair) {
+      chan_map_kernel<f32x4, NIN, ACC, 1, 0, true, Op>
           <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
     } else {
-      chan_map_kernel<f32x4, NIN, ACC, 1, 0, Op>
+      chan_map_kernel<f32x4, NIN, ACC, 1, 0, false, Op>
           <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
     }
   } else {
-    chan_map_kernel<float, NIN, ACC, 4, 0, Op>
+    chan_map_kernel<float, NIN, ACC, 4, 0, false, Op>
         <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out);
   }
   note_launch(symbol);

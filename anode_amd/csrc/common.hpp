@@ -169,6 +169,7 @@ struct Tuning {
   int nontemporal;        // bit 0: non-temporal stores, bit 1: non-temporal loads (streaming maps)
   int reduce_nontemporal; // bit 1: non-temporal loads in the reductions
   int nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
+  int reduce_min_tile;    // fewest elements a reduction tile reads (bounds the share of the per-tile epilogue)
 };
 
 // The non-temporal mask to use for an array of `bytes` bytes.

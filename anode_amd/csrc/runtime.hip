@@ -32,6 +32,7 @@ Tuning g_tuning = {
     /*nontemporal=*/3,
     /*reduce_nontemporal=*/2,
     /*nt_min_bytes=*/192 << 20,
+    /*reduce_min_tile=*/16384,
 };
 
 }  // namespace
@@ -114,7 +115,8 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
   // elements a tile aims to read: enough tiles to fill the chip, but never so
   // small that the per-tile epilogue dominates
   uint64_t per_tile = total / (wg_target ? wg_target : 1);
-  if (per_tile < 16384) per_tile = 16384;
+  const uint64_t floor_elems = g_tuning.reduce_min_tile > 0 ? uint64_t(g_tuning.reduce_min_tile) : 1;
+  if (per_tile < floor_elems) per_tile = floor_elems;
 
   if (S > kTilePos) {
     p.whole = 0;
@@ -216,7 +218,7 @@ ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int 
 ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return anode::FastDiv(d).div(n); }
 
 // Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal,
-// 4 reduce_nontemporal, 5 nt_min_bytes.
+// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile.
 // Returns the previous value, or -1 for an unknown knob.  A negative value
 // only reads.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
@@ -229,6 +231,7 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 3: slot = &t.nontemporal; break;
     case 4: slot = &t.reduce_nontemporal; break;
     case 5: slot = &t.nt_min_bytes; break;
+    case 6: slot = &t.reduce_min_tile; break;
     default: return -1;
   }
   const int old = *slot;
