@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -86,6 +87,49 @@ class PinnedBuffer {
   size_t n_ = 0;
 };
 
+// Owning handles, so that a constructor that throws half-way leaks nothing.
+template <typename T>
+class DeviceBuffer {
+ public:
+  explicit DeviceBuffer(size_t count) {
+    detail::hip_ok(hipMalloc(reinterpret_cast<void **>(&p_), (count ? count : 1) * sizeof(T)), "hipMalloc");
+  }
+  ~DeviceBuffer() { (void)hipFree(p_); }
+  DeviceBuffer(const DeviceBuffer &) = delete;
+  DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+  T *data() const { return p_; }
+
+ private:
+  T *p_ = nullptr;
+};
+
+class Event {
+ public:
+  Event() { detail::hip_ok(hipEventCreateWithFlags(&e_, hipEventDisableTiming), "hipEventCreate"); }
+  ~Event() { (void)hipEventDestroy(e_); }
+  Event(const Event &) = delete;
+  Event &operator=(const Event &) = delete;
+  hipEvent_t get() const { return e_; }
+
+ private:
+  hipEvent_t e_ = nullptr;
+};
+
+class CopyStream {  // default priority, does not synchronise with the null stream
+ public:
+  CopyStream() { detail::hip_ok(hipStreamCreateWithFlags(&s_, hipStreamNonBlocking), "hipStreamCreate"); }
+  ~CopyStream() {
+    (void)hipStreamSynchronize(s_);
+    (void)hipStreamDestroy(s_);
+  }
+  CopyStream(const CopyStream &) = delete;
+  CopyStream &operator=(const CopyStream &) = delete;
+  hipStream_t get() const { return s_; }
+
+ private:
+  hipStream_t s_ = nullptr;
+};
+
 // ---------------------------------------------------------------------------
 // u8 image batches in: copy stream + fused dequantize / normalise
 // ---------------------------------------------------------------------------
@@ -102,67 +146,58 @@ class ImageBatchStager {
       : inner_(inner), channels_(channels), batch_(batch), bytes_(inner * channels * batch) {
     if (depth < 1) throw std::invalid_argument("ImageBatchStager: depth must be at least 1");
     (void)sz2uint(bytes_);
-    detail::hip_ok(hipStreamCreateWithFlags(&copy_stream_, hipStreamNonBlocking), "hipStreamCreate");
-    slots_.resize(size_t(depth));
-    for (Slot &s : slots_) {
-      s.host = new PinnedBuffer<uint8_t>(bytes_);
-      detail::hip_ok(hipMalloc(reinterpret_cast<void **>(&s.dev), bytes_ ? bytes_ : 1), "hipMalloc");
-      detail::hip_ok(hipEventCreateWithFlags(&s.copied, hipEventDisableTiming), "hipEventCreate");
-      detail::hip_ok(hipEventCreateWithFlags(&s.consumed, hipEventDisableTiming), "hipEventCreate");
-    }
+    for (int i = 0; i < depth; ++i) slots_.push_back(std::make_unique<Slot>(bytes_));
   }
   ~ImageBatchStager() {
-    (void)hipStreamSynchronize(copy_stream_);
-    for (Slot &s : slots_) {
-      if (s.in_flight) (void)hipEventSynchronize(s.consumed);
-      (void)hipEventDestroy(s.copied);
-      (void)hipEventDestroy(s.consumed);
-      (void)hipFree(s.dev);
-      delete s.host;
+    // copies into the device slots and conversions still reading them finish before the slots are freed
+    (void)hipStreamSynchronize(copy_stream_.get());
+    for (auto &s : slots_) {
+      if (s->in_flight) (void)hipEventSynchronize(s->consumed.get());
     }
-    (void)hipStreamDestroy(copy_stream_);
   }
   ImageBatchStager(const ImageBatchStager &) = delete;
   ImageBatchStager &operator=(const ImageBatchStager &) = delete;
 
   int depth() const { return int(slots_.size()); }
   size_t batch_bytes() const { return bytes_; }
-  uint8_t *host_slot(int i) { return slots_.at(size_t(i)).host->data(); }
+  uint8_t *host_slot(int i) { return slots_.at(size_t(i))->host.data(); }
 
   // Blocks the host until slot i's previous copy has left the pinned buffer (it may then be refilled).
   void wait_slot_free(int i) {
-    Slot &s = slots_.at(size_t(i));
-    if (s.in_flight) detail::hip_ok(hipEventSynchronize(s.copied), "wait_slot_free");
+    Slot &s = *slots_.at(size_t(i));
+    if (s.in_flight) detail::hip_ok(hipEventSynchronize(s.copied.get()), "wait_slot_free");
   }
 
   // y[w, c, n] = fma(scale[c], float(q[w, c, n]), shift[c]); scale / shift are device arrays of `channels` floats.
   void submit(int i, const GPUDeviceConn &conn, const float *scale, const float *shift, DeviceArray<float> &y) {
-    Slot &s = slots_.at(size_t(i));
+    Slot &s = *slots_.at(size_t(i));
     detail::require_packed("ImageBatchStager::submit", y);
     if (y.shape.flat_len() != bytes_) throw std::invalid_argument("ImageBatchStager::submit: output size");
     hipStream_t compute = reinterpret_cast<hipStream_t>(conn.cuda_stream());
+    hipStream_t copy = copy_stream_.get();
     // the device slot may still be read by the conversion submitted from it last time
-    if (s.in_flight) detail::hip_ok(hipStreamWaitEvent(copy_stream_, s.consumed, 0), "hipStreamWaitEvent");
-    detail::hip_ok(hipMemcpyAsync(s.dev, s.host->data(), bytes_, hipMemcpyHostToDevice, copy_stream_), "hipMemcpyAsync");
-    detail::hip_ok(hipEventRecord(s.copied, copy_stream_), "hipEventRecord");
-    detail::hip_ok(hipStreamWaitEvent(compute, s.copied, 0), "hipStreamWaitEvent");
+    if (s.in_flight) detail::hip_ok(hipStreamWaitEvent(copy, s.consumed.get(), 0), "hipStreamWaitEvent");
+    detail::hip_ok(hipMemcpyAsync(s.dev.data(), s.host.data(), bytes_, hipMemcpyHostToDevice, copy), "hipMemcpyAsync");
+    detail::hip_ok(hipEventRecord(s.copied.get(), copy), "hipEventRecord");
+    detail::hip_ok(hipStreamWaitEvent(compute, s.copied.get(), 0), "hipStreamWaitEvent");
     anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(sz2uint(inner_), sz2uint(channels_), sz2uint(batch_), scale,
-                                                            shift, s.dev, y.as_mut_dptr(), conn.cuda_kernel_config(),
-                                                            conn.cuda_stream());
-    detail::hip_ok(hipEventRecord(s.consumed, compute), "hipEventRecord");
+                                                            shift, s.dev.data(), y.as_mut_dptr(),
+                                                            conn.cuda_kernel_config(), conn.cuda_stream());
+    detail::hip_ok(hipEventRecord(s.consumed.get(), compute), "hipEventRecord");
     s.in_flight = true;
   }
 
  private:
   struct Slot {
-    PinnedBuffer<uint8_t> *host = nullptr;
-    uint8_t *dev = nullptr;
-    hipEvent_t copied = nullptr, consumed = nullptr;
+    explicit Slot(size_t bytes) : host(bytes), dev(bytes) {}
+    PinnedBuffer<uint8_t> host;
+    DeviceBuffer<uint8_t> dev;
+    Event copied, consumed;
     bool in_flight = false;
   };
   size_t inner_, channels_, batch_, bytes_;
-  hipStream_t copy_stream_ = nullptr;
-  std::vector<Slot> slots_;
+  CopyStream copy_stream_;
+  std::vector<std::unique_ptr<Slot>> slots_;
 };
 
 // ---------------------------------------------------------------------------
@@ -171,10 +206,7 @@ class ImageBatchStager {
 
 class LogitsArgMaxReader {
  public:
-  explicit LogitsArgMaxReader(size_t max_rows) : host_(max_rows), rows_(max_rows) {
-    detail::hip_ok(hipMalloc(reinterpret_cast<void **>(&dev_), (max_rows ? max_rows : 1) * sizeof(uint32_t)), "hipMalloc");
-  }
-  ~LogitsArgMaxReader() { (void)hipFree(dev_); }
+  explicit LogitsArgMaxReader(size_t max_rows) : host_(max_rows), dev_(max_rows), rows_(max_rows) {}
   LogitsArgMaxReader(const LogitsArgMaxReader &) = delete;
   LogitsArgMaxReader &operator=(const LogitsArgMaxReader &) = delete;
 
@@ -185,16 +217,16 @@ class LogitsArgMaxReader {
     if (rows > rows_) throw std::invalid_argument("LogitsArgMaxReader::read: more rows than the reader was built for");
     const size_t K = rows ? logits.shape.flat_len() / rows : 0;
     hipStream_t s = reinterpret_cast<hipStream_t>(conn.cuda_stream());
-    anode_gpu_arg_max_packed_u32(sz2uint(K), sz2uint(rows), logits.as_dptr(), dev_, conn.cuda_kernel_config(),
+    anode_gpu_arg_max_packed_u32(sz2uint(K), sz2uint(rows), logits.as_dptr(), dev_.data(), conn.cuda_kernel_config(),
                                  conn.cuda_stream());
-    detail::hip_ok(hipMemcpyAsync(host_.data(), dev_, rows * sizeof(uint32_t), hipMemcpyDeviceToHost, s), "hipMemcpyAsync");
+    detail::hip_ok(hipMemcpyAsync(host_.data(), dev_.data(), rows * sizeof(uint32_t), hipMemcpyDeviceToHost, s), "hipMemcpyAsync");
     detail::hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize");
     return host_.data();
   }
 
  private:
   PinnedBuffer<uint32_t> host_;
-  uint32_t *dev_ = nullptr;
+  DeviceBuffer<uint32_t> dev_;
   size_t rows_;
 };
 
