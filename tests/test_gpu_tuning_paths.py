@@ -1,0 +1,68 @@
+"""The code paths that the default launch policy reaches only at benchmark sizes, exercised at test sizes with the
+exact checks of the other GPU tests: the non-temporal kernel variants (policy threshold set to zero, so every
+array takes them) and the grid-stride loops (grid capped at one workgroup per compute unit, so every thread walks
+several groups).  Also the plain variants with the non-temporal policy switched off.
+"""
+import pytest
+
+import test_gpu_additive as T_add
+import test_gpu_batch_norm as T_bn
+import test_gpu_flat as T_flat
+import test_gpu_softmax as T_sm
+from anode_amd import gpu
+
+pytestmark = pytest.mark.gpu
+
+# knob numbers of anode_gpu_set_tuning: 0 workgroups per CU of a streaming map (0 = full grid), 3 / 4 non-temporal
+# masks of the maps / reductions, 5 smallest array that takes the non-temporal variants
+PROFILES = {
+    "nontemporal_everywhere": {5: 0},
+    "nontemporal_off": {3: 0, 4: 0},
+    "one_workgroup_per_cu": {0: 1},
+    "one_workgroup_per_cu_nontemporal": {0: 1, 5: 0},
+}
+
+
+@pytest.fixture(params=sorted(PROFILES))
+def tuned(request):
+    saved = {k: gpu.set_tuning(k, v) for k, v in PROFILES[request.param].items()}
+    yield request.param
+    for k, v in saved.items():
+        gpu.set_tuning(k, v)
+
+
+def test_batch_norm_under_tuning(tuned, oracle):
+    # 401 408 and 802 816 elements: more than one pass of a 256-workgroup grid; S odd; element-aligned pointers
+    for S, C, N in [(784, 16, 32), (12544, 4, 8), (49, 300, 4), (5001, 2, 3)]:
+        for offset in (0, 1):
+            T_bn.test_batch_norm_all_symbols(oracle, S, C, N, offset)
+
+
+def test_flat_maps_under_tuning(tuned, oracle):
+    for name in sorted(T_flat.MAPS):
+        T_flat.test_flat_maps(oracle, name)
+    T_flat.test_two_input_maps_and_in_place_backward(oracle)
+    T_flat.test_positive_clip_in_place_and_sign_rules(oracle)
+    T_flat.test_upcast(oracle)
+    T_flat.test_dequantize_all_codes_and_ragged_lengths(oracle, -1.0, 1.0)
+    T_flat.test_one_hot(oracle, 4096, 5, 2)
+    T_flat.test_f1_loss_and_bwd(oracle, 70000, 2, 2)
+
+
+def test_softmax_under_tuning(tuned, oracle):
+    for K, R in [(10, 4000), (1000, 256), (4096, 3), (40000, 1)]:
+        for name in T_sm.ROW_ENTRY_POINTS:
+            T_sm.test_softmax_rows(oracle, name, K, R)
+    T_sm.test_softmax_cat_nll_and_bwd_rows(oracle, 1000, 256)
+    for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3)]:
+        T_sm.test_softmax_nd_all_symbols(oracle, P, C, N)
+
+
+def test_additive_under_tuning(tuned, oracle):
+    T_add.test_arg_max_rows(oracle)
+    T_add.test_quantize_u8(oracle, -4.0, 4.0)
+    T_add.test_bcast_affine_family(oracle, 3136, 3, 40)
+    T_add.test_channel_sums_and_mean_var(oracle, 784, 16, 32)
+    for masked in (False, True):
+        T_add.test_fused_batch_norm_equals_the_launch_sequence(oracle, 784, 16, 32, masked)
+    T_add.test_fused_softmax_nd_nll_equals_the_two_launches(oracle, 2048, 19, 2)
