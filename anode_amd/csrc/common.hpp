@@ -89,7 +89,12 @@ __device__ inline V load_stream(const V *p) {
 
 template <int NT, typename V>
 __device__ inline void store_stream(V *p, V v) {
-  if constexpr ((NT & kNtStore) != 0) {
+  if constexpr ((NT & kNtStore) != 0 && sizeof(V) == 16) {
+    // `nt` together with device scope (`sc1`: the line is written through instead of lingering dirty in the XCD's
+    // L2): measured 6.72 TB/s against 6.60 TB/s for `nt` alone on an 822 MB copy.  The builtin cannot express the
+    // pair, hence the instruction itself; it is an ordinary vector store.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(v) : "memory");
+  } else if constexpr ((NT & kNtStore) != 0) {
     __builtin_nontemporal_store(v, p);
   } else {
     *p = v;
