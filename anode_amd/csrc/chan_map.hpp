@@ -157,19 +157,16 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
   if (vec) {
     const uint32_t groups = len / 4, tail = len % 4;
     const bool pair = S >= 4 && S < 4096;
-    if (nt && pair) {
-      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, true, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
-    } else if (nt) {
-      chan_map_kernel<f32x4, NIN, ACC, 1, kNtLoad | kNtStore, false, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
-    } else if (pair) {
-      chan_map_kernel<f32x4, NIN, ACC, 1, 0, true, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
-    } else {
-      chan_map_kernel<f32x4, NIN, ACC, 1, 0, false, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
-    }
+    with_stream_policy(nt, [&](auto policy) {
+      constexpr int NT = decltype(policy)::value;
+      if (pair) {
+        chan_map_kernel<f32x4, NIN, ACC, 1, NT, true, Op>
+            <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+      } else {
+        chan_map_kernel<f32x4, NIN, ACC, 1, NT, false, Op>
+            <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+      }
+    });
   } else {
     chan_map_kernel<float, NIN, ACC, 4, 0, false, Op>
         <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out);

@@ -8,6 +8,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <mutex>
+#include <type_traits>
 
 // Layout fixed by the reference (routines_gpu/common.cuh:65-66, src/ffi.rs:28-33).
 struct KernelConfig {
@@ -77,6 +78,19 @@ struct FastDiv {
 // non-temporal access to the same address is folded into one ordinary access
 // by the compiler.
 constexpr int kNtStore = 1, kNtLoad = 2;
+
+// Runs f(std::integral_constant<int, NT>{}) for a policy value chosen at run time (stream_policy()): nothing,
+// streaming stores only, or streaming loads and stores.
+template <typename F>
+inline void with_stream_policy(int nt, F &&f) {
+  if (nt == (kNtLoad | kNtStore)) {
+    f(std::integral_constant<int, kNtLoad | kNtStore>{});
+  } else if (nt == kNtStore) {
+    f(std::integral_constant<int, kNtStore>{});
+  } else {
+    f(std::integral_constant<int, 0>{});
+  }
+}
 
 template <int NT, typename V>
 __device__ inline V load_stream(const V *p) {
@@ -175,9 +189,11 @@ struct Tuning {
   int reduce_nontemporal; // bit 1: non-temporal loads in the reductions
   int nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
   int reduce_min_tile;    // fewest elements a reduction tile reads (bounds the share of the per-tile epilogue)
+  int nt_store_min_bytes; // arrays of at least this size are written with streaming stores (never above nt_min_bytes)
 };
 
-// The non-temporal mask to use for an array of `bytes` bytes.
+// The streaming mask to use for an array of `bytes` bytes: the load bit of `mask` from nt_min_bytes on, the store
+// bit from nt_store_min_bytes on.
 int stream_policy(size_t bytes, int mask);
 Tuning &tuning();
 

@@ -123,11 +123,10 @@ void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, co
   if (vec) {
     // one 16-byte group per thread: measured faster on MI355X than any unrolled persistent loop
     const uint32_t groups = len / 4, tail = len % 4;
-    if (nt) {
-      flat_map_kernel<f32x4, NIN, 1, kNtLoad | kNtStore, Op><<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out);
-    } else {
-      flat_map_kernel<f32x4, NIN, 1, 0, Op><<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out);
-    }
+    with_stream_policy(nt, [&](auto policy) {
+      flat_map_kernel<f32x4, NIN, 1, decltype(policy)::value, Op>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out);
+    });
   } else {
     flat_map_kernel<float, NIN, 4, 0, Op><<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, op, a, b, out);
   }
@@ -206,11 +205,9 @@ void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, 
     const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
     // two groups per thread: with 4-byte loads a thread needs more than one in flight (41 us against 44 us at
     // [256,3,224,224])
-    if (nt) {
-      widen_u8x4_kernel<2, kNtLoad | kNtStore, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, x, y);
-    } else {
-      widen_u8x4_kernel<2, 0, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, x, y);
-    }
+    with_stream_policy(nt, [&](auto policy) {
+      widen_u8x4_kernel<2, decltype(policy)::value, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, x, y);
+    });
   } else {
     widen_u8_scalar_kernel<Op><<<stream_grid(len, 1), kBlock, 0, s>>>(len, op, x, y);
   }

@@ -33,6 +33,7 @@ Tuning g_tuning = {
     /*reduce_nontemporal=*/2,
     /*nt_min_bytes=*/192 << 20,
     /*reduce_min_tile=*/16384,
+    /*nt_store_min_bytes=*/16 << 20,
 };
 
 }  // namespace
@@ -63,7 +64,13 @@ uint32_t stream_grid(uint64_t work_items, int items_per_thread) {
 }
 
 int stream_policy(size_t bytes, int mask) {
-  return bytes >= size_t(g_tuning.nt_min_bytes > 0 ? g_tuning.nt_min_bytes : 0) ? mask : 0;
+  const size_t load_min = size_t(g_tuning.nt_min_bytes > 0 ? g_tuning.nt_min_bytes : 0);
+  size_t store_min = size_t(g_tuning.nt_store_min_bytes > 0 ? g_tuning.nt_store_min_bytes : 0);
+  if (store_min > load_min) store_min = load_min;
+  int out = 0;
+  if (bytes >= load_min) out |= mask & 2;   // kNtLoad
+  if (bytes >= store_min) out |= mask & 1;  // kNtStore
+  return out;
 }
 
 void require_pow2_block(const KernelConfig *cfg, const char *symbol) {
@@ -218,7 +225,7 @@ ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int 
 ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return anode::FastDiv(d).div(n); }
 
 // Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal,
-// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile.
+// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes.
 // Returns the previous value, or -1 for an unknown knob.  A negative value
 // only reads.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
@@ -232,6 +239,7 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 4: slot = &t.reduce_nontemporal; break;
     case 5: slot = &t.nt_min_bytes; break;
     case 6: slot = &t.reduce_min_tile; break;
+    case 7: slot = &t.nt_store_min_bytes; break;
     default: return -1;
   }
   const int old = *slot;

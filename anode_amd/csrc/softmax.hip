@@ -330,10 +330,10 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
 #define ANODE_ROW_WAVE(VPL)                                                              \
   do {                                                                                   \
-    if (vec && nt) {                                                                     \
-      softmax_row_wave_kernel<VPL, true, kNtLoad | kNtStore><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
-    } else if (vec) {                                                                    \
-      softmax_row_wave_kernel<VPL, true, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);       \
+    if (vec) {                                                                           \
+      with_stream_policy(nt, [&](auto policy) {                                          \
+        softmax_row_wave_kernel<VPL, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+      });                                                                                \
     } else {                                                                             \
       softmax_row_wave_kernel<VPL, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);      \
     }                                                                                    \
@@ -353,10 +353,10 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
 #define ANODE_ROW_BLOCKREG(VPT)                                                          \
   do {                                                                                   \
-    if (vec && nt) {                                                                     \
-      softmax_row_blockreg_kernel<VPT, true, kNtLoad | kNtStore><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
-    } else if (vec) {                                                                    \
-      softmax_row_blockreg_kernel<VPT, true, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);   \
+    if (vec) {                                                                           \
+      with_stream_policy(nt, [&](auto policy) {                                          \
+        softmax_row_blockreg_kernel<VPT, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+      });                                                                                \
     } else {                                                                             \
       softmax_row_blockreg_kernel<VPT, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);  \
     }                                                                                    \
@@ -651,8 +651,10 @@ void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, f
   // the input is streamed; the probabilities are read again by the NLL gather and the backward pass, so they
   // keep the default policy unless they are far larger than the last-level cache
   const size_t bytes = size_t(P) * C * N * sizeof(float);
-  if (PixVec<V>::W == 4 && stream_policy(bytes, tuning().nontemporal)) {
-    launch_softmax_nd_reg_nt<V, NLL, kNtLoad | kNtStore>(P, C, N, x, y, cat, nll, s);
+  if (PixVec<V>::W == 4) {
+    with_stream_policy(stream_policy(bytes, tuning().nontemporal), [&](auto policy) {
+      launch_softmax_nd_reg_nt<V, NLL, decltype(policy)::value>(P, C, N, x, y, cat, nll, s);
+    });
   } else {
     launch_softmax_nd_reg_nt<V, NLL, 0>(P, C, N, x, y, cat, nll, s);
   }
@@ -738,12 +740,10 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   if (vec) {
     const PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
-    if (stream_policy(size_t(len) * sizeof(float), tuning().nontemporal)) {
-      softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, kNtLoad | kNtStore>
+    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
+      softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, decltype(policy)::value>
           <<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
-    } else {
-      softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
-    }
+    });
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, 1, ignore);
     softmax_nd_cat_nll_bwd_kernel<float, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);

@@ -14,9 +14,11 @@ from anode_amd import gpu
 pytestmark = pytest.mark.gpu
 
 # knob numbers of anode_gpu_set_tuning: 0 workgroups per CU of a streaming map (0 = full grid), 3 / 4 non-temporal
-# masks of the maps / reductions, 5 smallest array that takes the non-temporal variants
+# masks of the maps / reductions, 5 smallest array read with non-temporal loads, 7 smallest array written with
+# streaming stores (the variants with streaming stores only sit between the two)
 PROFILES = {
     "nontemporal_everywhere": {5: 0},
+    "streaming_stores_only": {7: 0},
     "nontemporal_off": {3: 0, 4: 0},
     "one_workgroup_per_cu": {0: 1},
     "one_workgroup_per_cu_nontemporal": {0: 1, 5: 0},
