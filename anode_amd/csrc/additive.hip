@@ -101,6 +101,7 @@ struct FlatMultMap {
 // u8 codes -> per-channel affine f32: y = fma(scale[b], float(q), shift[b]).
 // Each lane loads one dword (4 codes) and stores 16 bytes; the channel of the
 // group's first code is found by exact division, then advanced incrementally.
+template <int NT>
 __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t n_groups, uint32_t tail,
                                                                        FastDiv div_s, FastDiv div_c,
                                                                        const float *__restrict__ scale,
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t 
         b = shift[c];
       }
     }
-    y4[g] = r;
+    store_stream<NT>(&y4[g], r);
   }
   if (blockIdx.x == 0 && threadIdx.x < tail) {
     const uint32_t i = n_groups * 4u + threadIdx.x;
@@ -415,7 +416,10 @@ ANODE_EXPORT void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32
   const FastDiv div_s(inner_dim), div_c(bcast_dim);
   if (aligned4(x) && aligned16(y)) {
     const uint32_t groups = len / 4, tail = len % 4;
-    bcast_dequantize_u8x4_kernel<<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, scale, shift, x, y);
+    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
+      bcast_dequantize_u8x4_kernel<decltype(policy)::value>
+          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, scale, shift, x, y);
+    });
   } else {
     bcast_dequantize_u8_scalar_kernel<<<stream_grid(len, 1), kBlock, 0, s>>>(len, div_s, div_c, scale, shift, x, y);
   }

@@ -11,7 +11,7 @@ namespace {
 // discrete.cu:21-46  y[p,k,n] = (label[p + P*n] == k) ? 1 : 0 over a packed
 // [P, K, N] output.  A thread reads the labels of W consecutive pixels once and
 // writes their K outputs, 16 bytes per store, coalesced across the wave.
-template <int W>
+template <int W, int NT>
 __global__ __launch_bounds__(kBlock) void one_hot_kernel(uint32_t P, uint32_t K, uint32_t total_groups,
                                                          FastDiv div_gps, const uint32_t *__restrict__ cat,
                                                          float *__restrict__ y) {
@@ -33,7 +33,7 @@ __global__ __launch_bounds__(kBlock) void one_hot_kernel(uint32_t P, uint32_t K,
       } else {
         v = (lab == k) ? 1.0f : 0.0f;
       }
-      *reinterpret_cast<V *>(y + base + size_t(P) * k) = v;
+      store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(P) * k), v);
     }
   }
 }
@@ -83,10 +83,11 @@ ANODE_EXPORT void anode_gpu_discrete_one_hot_3d1_packed_f32(uint32_t dim0, uint3
   hipStream_t s = as_stream(stream);
   if (dim0 % 4 == 0 && aligned16(x) && aligned16(y)) {
     const uint32_t gps = dim0 / 4, total = gps * dim2;
-    one_hot_kernel<4><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(gps), x, y);
+    // ordinary stores: with streaming stores this kernel, which writes K planes per thread, measured 15 % slower
+    one_hot_kernel<4, 0><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(gps), x, y);
   } else {
     const uint32_t total = dim0 * dim2;
-    one_hot_kernel<1><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(dim0), x, y);
+    one_hot_kernel<1, 0><<<stream_grid(total, 1), kBlock, 0, s>>>(dim0, cat_dim1, total, FastDiv(dim0), x, y);
   }
   note_launch(__func__);
 }

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
 // they are copied to LDS with full-width coalesced loads (row pitch K|1, so that threads reading their own row hit
 // distinct banks), each thread normalises its row in registers, and the tile goes back the same way.  No cross-lane
 // traffic at all, which is what bounds the lane-group kernel below for short rows.
-template <int KMAX>
+template <int KMAX, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, FastDiv div_k, int vec,
                                                                  const float *__restrict__ x,
                                                                  float *__restrict__ y) {
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
           ++q;
         }
       }
-      reinterpret_cast<f32x4 *>(yt)[g] = v;
+      store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, v);
     }
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
       uint32_t q, c;
@@ -308,15 +308,18 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     const size_t lds_bytes = size_t(kBlock) * (K | 1u) * sizeof(float);
     const FastDiv div_k(K);
     const int vec = (aligned16(x) && aligned16(y)) ? 1 : 0;
-    if (K <= 4) {
-      softmax_row_lds_kernel<4><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
-    } else if (K <= 8) {
-      softmax_row_lds_kernel<8><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
-    } else if (K <= 16) {
-      softmax_row_lds_kernel<16><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
-    } else {
-      softmax_row_lds_kernel<32><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
-    }
+    with_stream_policy(nt & kNtStore, [&](auto policy) {
+      constexpr int NT = decltype(policy)::value;
+      if (K <= 4) {
+        softmax_row_lds_kernel<4, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+      } else if (K <= 8) {
+        softmax_row_lds_kernel<8, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+      } else if (K <= 16) {
+        softmax_row_lds_kernel<16, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+      } else {
+        softmax_row_lds_kernel<32, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+      }
+    });
   } else if (K <= 64) {
     uint32_t log2g = 0;
     while ((1u << log2g) < K) ++log2g;
