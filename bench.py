@@ -333,6 +333,27 @@ def all_symbols(torch, gpu):
     return rows
 
 
+def graph_replay(torch, run_step, steps, step_bytes):
+    """The same step captured once as a HIP graph and replayed: what the launch gaps cost (reported beside `value`,
+    which stays the plainly launched figure)."""
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run_step()  # the reductions' scratch for this stream exists before capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run_step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    g_s = (time.perf_counter() - t0) / steps
+    return {"ms_per_step": round(g_s * 1e3, 4), "gbps": round(step_bytes / g_s / 1e9, 1),
+            "pct_of_hbm_peak": round(100 * step_bytes / g_s / 1e9 / HBM_PEAK_GBPS, 2)}
+
+
 def small_shape_latency(torch, gpu, groups, passes=100):
     """Launch-bound shapes (config 0, config 3a): time per pass over `passes` back-to-back passes, launched one entry
     point at a time and as one captured HIP graph replayed.  Separates launch latency from bandwidth."""
@@ -650,27 +671,20 @@ def main():
         "per_symbol": per_symbol,
     }
     if not only:
-        # the same step captured once as a HIP graph and replayed: what the launch gaps cost (reported beside `value`,
-        # which stays the plainly launched figure)
-        side = torch.cuda.Stream()
-        with torch.cuda.stream(side):
-            run_step()  # the reductions' scratch for this stream exists before capture
-        side.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            run_step()
-        graph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        g_s = (time.perf_counter() - t0) / args.steps
-        out["graph_replay"] = {"ms_per_step": round(g_s * 1e3, 4), "gbps": round(step_bytes / g_s / 1e9, 1),
-                               "pct_of_hbm_peak": round(100 * step_bytes / g_s / 1e9 / HBM_PEAK_GBPS, 2)}
-        out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches))
+        # side measurements: a failure in one of them is recorded and must not cost the headline line
+        try:
+            out["graph_replay"] = graph_replay(torch, run_step, args.steps, step_bytes)
+        except Exception as e:  # noqa: BLE001
+            out["graph_replay"] = {"error": repr(e)}
+        try:
+            out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches))
+        except Exception as e:  # noqa: BLE001
+            out["small_shapes"] = {"error": repr(e)}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        try:
+            out["cpu_baseline"] = cpu_baseline()
+        except Exception as e:  # noqa: BLE001
+            out["cpu_baseline"] = {"error": repr(e)}
     print(json.dumps(out), flush=True)
 
 
