@@ -187,7 +187,7 @@ struct MeanVarReduce {
     s1 = fma(d, d, s1);
   }
   __device__ void finalize(uint32_t c, double s0, double s1, double) const {
-    const double k = double(x[size_t(c) * S]);
+    const double k = n > 0.0 ? double(x[size_t(c) * S]) : 0.0;  // an empty array has no first element to read
     mean[c] = float(k + s0 / n);
     var[c] = float((s1 - s0 * s0 / n) / n + eps);
   }

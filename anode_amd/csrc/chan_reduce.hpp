@@ -309,12 +309,43 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_fold_block_kernel(uint32_t
   if (threadIdx.x == 0) op.finalize(c, s0, s1, s2);
 }
 
+// Caller-provided partial-sum buffer for launch_chan_reduce (instead of the per-stream cache, which allocates).
+struct FixedScratch {
+  void *ptr;
+  size_t bytes;
+};
+
+// Bytes of partial sums a reduction with NACC sums needs for plan `pl` (0 when every channel has one partial).
+inline size_t chan_reduce_scratch_bytes(const ReducePlan &pl, int nacc) {
+  return pl.ppc > 1 ? size_t(nacc) * pl.C * pl.ppc * sizeof(double) : 0;
+}
+
+// Status of launch_chan_reduce.  The reference ABI is void: its entry points drop the status, which is also
+// recorded for anode_gpu_take_last_error().
+enum ReduceStatus : int {
+  kReduceOk = 0,
+  kReduceScratchTooSmall = 1,   // the caller-provided buffer cannot hold the partial sums; nothing was enqueued
+  kReduceScratchUnavailable = 2 // the per-stream buffer could not be provided; nothing was enqueued
+};
+
+// `fixed` (optional) replaces the per-stream scratch cache: with it the call allocates nothing.
 template <typename Op>
-void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
-                        const float *b, CUstream_st *stream, const float *c = nullptr) {
+int launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op op, const float *a,
+                       const float *b, CUstream_st *stream, const float *c = nullptr,
+                       const FixedScratch *fixed = nullptr) {
   const uint32_t len = checked_len(S, C, N, symbol);
-  if (len == 0) return;
   hipStream_t s = as_stream(stream);
+  if (len == 0) {
+    // No element to add, but every channel still gets its finalised value (0/0 = NaN for a mean, the
+    // accumulate twins add their term of an empty sum), as in the reference, whose one block per channel
+    // always writes its output (e.g. routines_gpu/batch_norm.cu:52-56).
+    if (C > 0) {
+      const uint32_t waves_per_block = kBlock / kWave;
+      chan_reduce_fold_kernel<Op><<<(C + waves_per_block - 1) / waves_per_block, kBlock, 0, s>>>(C, 0, op, nullptr);
+      note_launch(symbol);
+    }
+    return kReduceOk;
+  }
   const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b)) && (Op::NIN < 3 || aligned16(c));
   const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
   if (Op::NIN < 2) b = a;
@@ -323,9 +354,16 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
 
   ScratchLease lease{nullptr, std::unique_lock<std::mutex>()};
   double *part = nullptr;
-  if (pl.ppc > 1) {
-    lease = acquire_scratch(s, size_t(Op::NACC) * C * pl.ppc * sizeof(double));
-    part = static_cast<double *>(lease.ptr);
+  const size_t need = chan_reduce_scratch_bytes(pl, Op::NACC);
+  if (need > 0) {
+    if (fixed) {
+      if (need > fixed->bytes) return kReduceScratchTooSmall;
+      part = static_cast<double *>(fixed->ptr);
+    } else {
+      lease = acquire_scratch(s, need, symbol);
+      if (!lease.ptr) return kReduceScratchUnavailable;
+      part = static_cast<double *>(lease.ptr);
+    }
   }
   if (pl.whole) {
     const FastDiv div_s(S);
@@ -359,6 +397,7 @@ void launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, 
     }
     note_launch(symbol);
   }
+  return kReduceOk;
 }
 
 #endif  // __HIPCC__

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 #include <mutex>
@@ -180,16 +181,21 @@ __device__ inline float block_max(float v, float *lds) {
 int device_cu_count();
 
 // Tunable launch parameters; defaults are set in runtime.hip and may be
-// changed at run time through anode_gpu_set_tuning().
+// changed at run time through anode_gpu_set_tuning() (a test and measurement
+// hook, not part of the operator ABI).  Each knob is an atomic read with
+// relaxed order, so that a host thread may change one while others launch.
+struct Knob {
+  std::atomic<int> v;
+  operator int() const { return v.load(std::memory_order_relaxed); }
+};
 struct Tuning {
-  int flat_wg_per_cu;     // workgroups per CU of a streaming map; 0 = one 16-byte group per thread (full grid)
-  int flat_unroll;        // unused (kept so that knob numbers stay stable)
-  int reduce_wg_target;   // workgroups a per-channel reduction aims to launch
-  int nontemporal;        // bit 0: non-temporal stores, bit 1: non-temporal loads (streaming maps)
-  int reduce_nontemporal; // bit 1: non-temporal loads in the reductions
-  int nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
-  int reduce_min_tile;    // fewest elements a reduction tile reads (bounds the share of the per-tile epilogue)
-  int nt_store_min_bytes; // arrays of at least this size are written with streaming stores (never above nt_min_bytes)
+  Knob flat_wg_per_cu;     // workgroups per CU of a streaming map; 0 = one 16-byte group per thread (full grid)
+  Knob reduce_wg_target;   // workgroups a per-channel reduction aims to launch
+  Knob nontemporal;        // bit 0: non-temporal stores, bit 1: non-temporal loads (streaming maps); 0, 1 or 3
+  Knob reduce_nontemporal; // bit 1: non-temporal loads in the reductions
+  Knob nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
+  Knob reduce_min_tile;    // fewest elements a reduction tile reads (bounds the share of the per-tile epilogue)
+  Knob nt_store_min_bytes; // arrays of at least this size are written with streaming stores (never above nt_min_bytes)
 };
 
 // The streaming mask to use for an array of `bytes` bytes: the load bit of `mask` from nt_min_bytes on, the store
@@ -211,18 +217,23 @@ void require_pow2_block(const KernelConfig *cfg, const char *symbol);
 // fit (the reference's callers guard this: src/ops_gpu.rs:57-61).
 uint32_t checked_len(uint64_t a, uint64_t b, uint64_t c, const char *symbol);
 
-// Records the status of the launch just made (hipGetLastError) for
-// anode_gpu_take_last_error() and prints it to stderr on failure.
+// Looks at the thread's HIP error state after a launch (hipPeekAtLastError: the state is left to the caller) and,
+// when an error has appeared, records it for anode_gpu_take_last_error() and prints it to stderr.
 void note_launch(const char *symbol);
+// Records `e` for anode_gpu_take_last_error() and prints "<symbol>: <what>: <error string>".
+void note_error(const char *symbol, hipError_t e, const char *what);
 
 // A device buffer private to (current device, stream), grown on demand and
-// kept for the life of the process.  The lease holds the cache's lock: keep it
+// kept until anode_gpu_release_scratch().  The lease holds the cache's lock: keep it
 // alive until every kernel that uses the buffer has been enqueued, so that two
-// host threads sharing a stream cannot interleave their launches.
+// host threads sharing a stream cannot interleave their launches.  When the
+// buffer cannot be provided (allocation failure, or the stream is being captured
+// and would have to allocate) the error is recorded under `symbol`, ptr is null
+// and the lock is not held: the caller skips its launch.
 struct ScratchLease {
   void *ptr;
   std::unique_lock<std::mutex> lock;
 };
-ScratchLease acquire_scratch(hipStream_t stream, size_t bytes);
+ScratchLease acquire_scratch(hipStream_t stream, size_t bytes, const char *symbol);
 
 }  // namespace anode

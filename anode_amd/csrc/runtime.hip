@@ -9,6 +9,7 @@
 #include <cstring>
 #include <map>
 #include <utility>
+#include <vector>
 
 namespace anode {
 
@@ -21,19 +22,19 @@ std::atomic<int> g_last_error{0};
 struct ScratchBuf {
   void *ptr = nullptr;
   size_t cap = 0;
+  std::vector<void *> outgrown;  // earlier, smaller buffers: kernels in flight may still use them
 };
 std::mutex g_scratch_mutex;
 std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch;
 
 Tuning g_tuning = {
-    /*flat_wg_per_cu=*/0,
-    /*flat_unroll=*/1,
-    /*reduce_wg_target=*/8192,
-    /*nontemporal=*/3,
-    /*reduce_nontemporal=*/2,
-    /*nt_min_bytes=*/192 << 20,
-    /*reduce_min_tile=*/16384,
-    /*nt_store_min_bytes=*/16 << 20,
+    /*flat_wg_per_cu=*/{{0}},
+    /*reduce_wg_target=*/{{8192}},
+    /*nontemporal=*/{{3}},
+    /*reduce_nontemporal=*/{{2}},
+    /*nt_min_bytes=*/{{192 << 20}},
+    /*reduce_min_tile=*/{{16384}},
+    /*nt_store_min_bytes=*/{{16 << 20}},
 };
 
 }  // namespace
@@ -93,11 +94,21 @@ uint32_t checked_len(uint64_t a, uint64_t b, uint64_t c, const char *symbol) {
 }
 
 void note_launch(const char *symbol) {
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
+  // Peek, never take: the thread's HIP error state belongs to the caller (the reference's kernels never touch
+  // the CUDA error state, so the host framework's own checks must keep seeing what they see today).  An error
+  // that was already pending at this thread's previous check is not reported again.
+  static thread_local hipError_t pending = hipSuccess;
+  const hipError_t e = hipPeekAtLastError();
+  if (e != hipSuccess && e != pending) {
     g_last_error.store(int(e), std::memory_order_relaxed);
-    std::fprintf(stderr, "%s: launch failed: %s\n", symbol, hipGetErrorString(e));
+    std::fprintf(stderr, "%s: HIP error pending after the launch: %s\n", symbol, hipGetErrorString(e));
   }
+  pending = e;
+}
+
+void note_error(const char *symbol, hipError_t e, const char *what) {
+  g_last_error.store(int(e), std::memory_order_relaxed);
+  std::fprintf(stderr, "%s: %s: %s; nothing was enqueued\n", symbol, what, hipGetErrorString(e));
 }
 
 namespace {
@@ -176,25 +187,35 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
   return p;
 }
 
-ScratchLease acquire_scratch(hipStream_t stream, size_t bytes) {
+ScratchLease acquire_scratch(hipStream_t stream, size_t bytes, const char *symbol) {
   ScratchLease lease{nullptr, std::unique_lock<std::mutex>(g_scratch_mutex)};
   int dev = 0;
   (void)hipGetDevice(&dev);
   ScratchBuf &buf = g_scratch[std::make_pair(dev, stream)];
   if (buf.cap < bytes) {
-    // Grow geometrically.  The previous buffer may still be read by kernels in
-    // flight on this stream, so it is not freed: it stays allocated until the
-    // process ends (bounded by the doubling).
+    // Growing means hipMalloc, which a stream under capture cannot take (it would fail and could invalidate the
+    // capture): refuse instead, and tell the caller how to avoid it.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+      note_error(symbol, hipErrorStreamCaptureUnsupported,
+                 "the stream is being captured and has no reduction scratch yet (call anode_gpu_reserve_scratch "
+                 "or run the entry point once on this stream before capturing)");
+      lease.lock.unlock();
+      return lease;
+    }
+    // Grow geometrically.  The previous buffer may still be read by kernels in flight on this stream, so it is
+    // not freed here; anode_gpu_release_scratch() frees everything a stream holds once the caller has
+    // synchronised it.
     size_t cap = buf.cap ? buf.cap : size_t(1) << 16;
     while (cap < bytes) cap <<= 1;
     void *p = nullptr;
     const hipError_t e = hipMalloc(&p, cap);
-    if (e != hipSuccess) {
-      g_last_error.store(int(e), std::memory_order_relaxed);
-      std::fprintf(stderr, "anode_routines_gpu: cannot allocate %zu bytes of reduction scratch: %s\n",
-                   cap, hipGetErrorString(e));
-      std::abort();
+    if (e != hipSuccess || !p) {
+      note_error(symbol, e != hipSuccess ? e : hipErrorOutOfMemory, "cannot allocate the reduction scratch");
+      lease.lock.unlock();
+      return lease;
     }
+    if (buf.ptr) buf.outgrown.push_back(buf.ptr);
     buf.ptr = p;
     buf.cap = cap;
   }
@@ -210,6 +231,39 @@ ANODE_EXPORT int anode_gpu_take_last_error(void) {
 
 ANODE_EXPORT uint32_t anode_gpu_reference_symbol_count(void) { return 46; }
 
+// Upper bound of the partial-sum bytes a reduction over [S, C, N] needs: three sums, either alignment.
+ANODE_EXPORT size_t anode_gpu_reduce_scratch_bytes(uint32_t S, uint32_t C, uint32_t N) {
+  const uint32_t target = uint32_t(anode::tuning().reduce_wg_target);
+  const size_t a = anode::chan_reduce_scratch_bytes(anode::plan_chan_reduce(S, C, N, true, target), 3);
+  const size_t b = anode::chan_reduce_scratch_bytes(anode::plan_chan_reduce(S, C, N, false, target), 3);
+  return a > b ? a : b;
+}
+
+// Makes sure that the reduction entry points find at least `bytes` of partial-sum scratch for `stream` on the
+// current device, so that later calls on that stream allocate nothing (needed before the stream is captured into a
+// HIP graph).  Returns 0 or the hipError_t of the failed allocation.
+ANODE_EXPORT int anode_gpu_reserve_scratch(CUstream_st *stream, size_t bytes) {
+  anode::ScratchLease lease = anode::acquire_scratch(anode::as_stream(stream), bytes, __func__);
+  if (lease.ptr || bytes == 0) return 0;
+  const int e = anode::g_last_error.load(std::memory_order_relaxed);
+  return e ? e : int(hipErrorOutOfMemory);
+}
+
+// Frees every scratch buffer held for `stream` on the current device.  The caller must have synchronised the
+// stream: kernels in flight would lose their partial sums.  Returns the number of buffers freed.
+ANODE_EXPORT int anode_gpu_release_scratch(CUstream_st *stream) {
+  std::lock_guard<std::mutex> lock(anode::g_scratch_mutex);
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const auto it = anode::g_scratch.find(std::make_pair(dev, anode::as_stream(stream)));
+  if (it == anode::g_scratch.end()) return 0;
+  int freed = 0;
+  for (void *p : it->second.outgrown) freed += (hipFree(p) == hipSuccess);
+  if (it->second.ptr) freed += (hipFree(it->second.ptr) == hipSuccess);
+  anode::g_scratch.erase(it);
+  return freed;
+}
+
 // Host-only view of the reduction tiling for a [S, C, N] array, as 12 words:
 // whole, CB, SB, n_ctiles, n_stiles, NB, n_ntiles, ppc, vec, grid, 0, 0.
 ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int ptrs_aligned,
@@ -224,16 +278,15 @@ ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int 
 // the kernels compute it.
 ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return anode::FastDiv(d).div(n); }
 
-// Knobs: 0 flat_wg_per_cu, 1 flat_unroll, 2 reduce_wg_target, 3 nontemporal,
-// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes.
-// Returns the previous value, or -1 for an unknown knob.  A negative value
-// only reads.
+// Test and measurement hook (not declared in the public header).  Knobs: 0 flat_wg_per_cu, 2 reduce_wg_target,
+// 3 nontemporal (0, 1 or 3: streaming loads without streaming stores is not a policy the maps are built for),
+// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes.  Returns the previous value; a
+// negative value only reads.  Returns -1, and changes nothing, for an unknown knob or a value the knob does not take.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
   anode::Tuning &t = anode::tuning();
-  int *slot = nullptr;
+  anode::Knob *slot = nullptr;
   switch (knob) {
     case 0: slot = &t.flat_wg_per_cu; break;
-    case 1: slot = &t.flat_unroll; break;
     case 2: slot = &t.reduce_wg_target; break;
     case 3: slot = &t.nontemporal; break;
     case 4: slot = &t.reduce_nontemporal; break;
@@ -242,7 +295,8 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 7: slot = &t.nt_store_min_bytes; break;
     default: return -1;
   }
+  if (knob == 3 && value >= 0 && value != 0 && value != 1 && value != 3) return -1;
   const int old = *slot;
-  if (value >= 0) *slot = value;
+  if (value >= 0) slot->v.store(value, std::memory_order_relaxed);
   return old;
 }

@@ -266,9 +266,26 @@ void anode_gpu_online_add_packed_f32(uint32_t len, float rate, const float *x, f
  * maximum starting from (-inf, 0); NaN never selected.  xs is a HOST pointer. */
 size_t anode_host_arg_max_f32(const float *xs, size_t len);
 
+/* The reduction scratch.  No reference counterpart: the reference reduces a channel in one block and needs no
+ * workspace; this library cuts a channel into tiles and keeps one fp64 partial sum per (channel, tile) in a device
+ * buffer per (device, stream), allocated by the first reduction call on that stream and grown on demand.  When the
+ * buffer cannot be provided -- allocation failure, or the stream is being captured into a HIP graph and holds no
+ * buffer that is large enough -- the reduction entry point enqueues nothing, reports on stderr and records the
+ * hipError_t for anode_gpu_take_last_error().  A HIP graph keeps the buffer of the stream it was captured on: graphs
+ * captured on one stream must not be replayed concurrently with each other or with eager reduction calls on that
+ * stream. */
+/* Upper bound of the scratch bytes any reduction entry point needs for a [dim0, dim1, dim2] array. */
+size_t anode_gpu_reduce_scratch_bytes(uint32_t dim0, uint32_t dim1, uint32_t dim2);
+/* Makes `stream` (current device) hold at least `bytes` of scratch, so that later calls allocate nothing (call it
+ * before capturing the stream).  Returns 0 or the hipError_t of the failed allocation. */
+int anode_gpu_reserve_scratch(struct CUstream_st *stream, size_t bytes);
+/* Frees the scratch of `stream` (current device); the caller has synchronised the stream.  Returns the number of
+ * buffers freed. */
+int anode_gpu_release_scratch(struct CUstream_st *stream);
+
 /* Library introspection.  No reference counterpart. */
 /* 0 when no launch made by this library has failed since the last call; otherwise the hipError_t
- * of the most recent failed launch.  Reading clears it. */
+ * of the most recent failure.  Reading clears it (the thread's own HIP error state is never cleared by this library). */
 int anode_gpu_take_last_error(void);
 /* Number of entry points of Part 1 (46). */
 uint32_t anode_gpu_reference_symbol_count(void);

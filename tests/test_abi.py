@@ -147,6 +147,50 @@ def test_reduction_entry_points_abort_on_non_power_of_two_block(name):
     assert "returned" not in r.stdout
 
 
+_NO_DEVICE_SNIPPET = r"""
+import ctypes, sys
+sys.path.insert(0, {root!r})
+from anode_amd import _lib
+lib = _lib.load()
+cfg = _lib.KernelConfig(1024, 1024)
+take = lib.symbol("anode_gpu_take_last_error")
+# with no device visible every allocation fails: a stand-in for an exhausted GPU that needs none
+rc = lib.symbol("anode_gpu_reserve_scratch")(None, 1 << 20)
+print("reserve", rc, take(), take())
+# [12544, 64, 256] needs partial sums: the reduction must give up, record the error and return
+lib.symbol("anode_gpu_batch_mean_3d1_packed_f32")(12544, 64, 256, None, None, ctypes.byref(cfg), None)
+print("mean", take(), take())
+print("released", lib.symbol("anode_gpu_release_scratch")(None))
+print("alive")
+"""
+
+
+def test_scratch_allocation_failure_is_reported_not_fatal():
+    # The ABI returns void: when the partial-sum buffer cannot be allocated the call must skip its launch, keep the
+    # process alive and leave the error for anode_gpu_take_last_error().  No GPU is involved: the child sees no device.
+    env = dict(os.environ, HIP_VISIBLE_DEVICES="", ROCR_VISIBLE_DEVICES="")
+    code = _NO_DEVICE_SNIPPET.format(root=_lib.REPO_ROOT)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120, env=env)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    out = dict((line.split()[0], line.split()[1:]) for line in r.stdout.splitlines() if line.strip())
+    rc, err, again = (int(v) for v in out["reserve"])
+    assert rc != 0 and err == rc and again == 0          # reported once, then cleared
+    err, again = (int(v) for v in out["mean"])
+    assert err != 0 and again == 0
+    assert out["released"] == ["0"] and "alive" in out
+    assert "cannot allocate the reduction scratch" in r.stderr and "nothing was enqueued" in r.stderr
+    assert "anode_gpu_batch_mean_3d1_packed_f32" in r.stderr
+
+
+def test_scratch_size_query_bounds_the_plan():
+    lib = _lib.load()
+    q = lib.symbol("anode_gpu_reduce_scratch_bytes")
+    for S, C, N in [(784, 16, 32), (12544, 64, 256), (49, 2048, 256), (1, 1000, 64), (3, 5, 7)]:
+        ppcs = [_plan(S, C, N, a)["ppc"] for a in (True, False)]
+        assert q(S, C, N) == max(3 * 8 * C * ppc if ppc > 1 else 0 for ppc in ppcs)  # three fp64 sums per partial
+    assert q(0, 5, 3) == 0 and q(7, 5, 1) == 0
+
+
 def test_host_arg_max_follows_the_reference_rule():
     # src/utils/mod.rs:31-41: start from (-inf, 0); strictly greater wins; NaN never wins
     fn = _lib.load().symbol("anode_host_arg_max_f32")

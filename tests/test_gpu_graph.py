@@ -5,6 +5,8 @@ and synchronisations between the replays; every replay must equal the eager resu
 The reductions keep their partial-sum buffer per (device, stream) and allocate it on first use, so the sequence is
 run once on the capture stream before capture (allocation is not possible while capturing).
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -79,3 +81,49 @@ def test_graph_replay_equals_eager(d):
         torch.cuda.synchronize()
         for got, want in zip(gb + gh, eb + eh):
             assert_bit_exact(host(got), host(want), f"replay with seed {seed}")
+
+
+def test_capture_without_scratch_is_refused_and_reserve_makes_it_work():
+    # A reduction whose channels are cut into several tiles needs the stream's partial-sum buffer.  Allocating it is
+    # impossible while the stream is being captured: the call must enqueue nothing, record
+    # hipErrorStreamCaptureUnsupported (900) and leave the capture valid.  After anode_gpu_reserve_scratch the same
+    # capture works and its replays equal the eager result.
+    from anode_amd import gpu
+    from anode_amd._lib import load
+
+    lib = load()
+    d = (12544, 8, 16)
+    S, C, N = d
+    g = np.random.default_rng(5)
+    x = dev((2 + 3 * g.standard_normal(S * C * N)).astype(F32))
+    mean, marker, want = empty(C), empty(4), empty(C)
+    stream = torch.cuda.Stream()
+    handle = ctypes.c_void_p(stream.cuda_stream)
+    stream.synchronize()
+    lib.symbol("anode_gpu_release_scratch")(handle)      # torch hands out pooled streams: drop what an earlier test left
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        marker.fill_(1.0)
+        gpu.call("anode_gpu_batch_mean_3d1_packed_f32", *d, x, mean)
+        err = gpu.take_last_error()
+    assert err == 900, err
+    graph.replay()
+    torch.cuda.synchronize()
+    assert np.all(host(marker) == 1.0) and np.all(np.isnan(host(mean)))   # the capture survived; nothing was enqueued
+
+    need = lib.symbol("anode_gpu_reduce_scratch_bytes")(*d)
+    assert need > 0
+    assert lib.symbol("anode_gpu_reserve_scratch")(handle, need) == 0
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2, stream=stream):
+        call("anode_gpu_batch_mean_3d1_packed_f32", *d, x, mean)
+    call("anode_gpu_batch_mean_3d1_packed_f32", *d, x, want)
+    for k in range(3):
+        mean.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert_bit_exact(host(mean), host(want), f"replay {k}")
+    stream.synchronize()
+    assert lib.symbol("anode_gpu_release_scratch")(handle) >= 1
