@@ -9,6 +9,8 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <cstdio>
+#include <mutex>
 
 namespace anode {
 namespace {
@@ -450,6 +452,68 @@ ANODE_EXPORT void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_
                                                           const KernelConfig *, CUstream_st *stream) {
   launch_chan_reduce(__func__, dim0, dim1, dim2,
                      MeanVarReduce{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)}, x, nullptr, stream);
+}
+
+// ---------------------------------------------------------------------------
+// batch_mean_var for callers that cannot allocate (code under HIP graph
+// capture, serving loops, harnesses that forbid hipMalloc): the partial sums
+// live in a device array that is part of the library's image, one copy per GPU.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr size_t kNoAllocScratchBytes = size_t(4) << 20;  // 4 MiB per GPU, held until the process ends
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_noalloc_mutex;
+void *g_noalloc_ptr[kNoAllocMaxDevices] = {};  // device address of `scratch` on each GPU, looked up once
+}  // namespace
+
+static __device__ __align__(256) double scratch[kNoAllocScratchBytes / sizeof(double)];
+
+// The device address of this GPU's copy of `scratch` (in host code the array's name is only a handle for the
+// symbol, not an address a kernel could use).  Looked up on the first call with each device current.
+static void *noalloc_scratch_of_current_device(const char *symbol) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kNoAllocMaxDevices) {
+    note_error(symbol, hipErrorInvalidDevice, "no current device to take the scratch array from");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (!g_noalloc_ptr[dev]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      note_error(symbol, e != hipSuccess ? e : hipErrorInvalidSymbol, "cannot look up the scratch array");
+      return nullptr;
+    }
+    g_noalloc_ptr[dev] = p;
+  }
+  return g_noalloc_ptr[dev];
+}
+
+ANODE_EXPORT int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                                 float epsilon, const float *x, float *mean,
+                                                                 float *var, const KernelConfig *,
+                                                                 CUstream_st *stream) {
+  // Sizes are checked before anything touches the device, so that a refusal has no side effect.
+  const bool ptrs_aligned = aligned16(x);
+  const ReducePlan pl = plan_chan_reduce(dim0, dim1, dim2, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
+  const size_t need = chan_reduce_scratch_bytes(pl, MeanVarReduce::NACC);
+  if (need > kNoAllocScratchBytes) {
+    std::fprintf(stderr,
+                 "%s: [%u, %u, %u] needs %zu bytes of partial sums, more than the %zu bytes of the static scratch "
+                 "array; use anode_gpu_batch_mean_var_3d1_packed_f32; nothing was enqueued\n",
+                 __func__, dim0, dim1, dim2, need, kNoAllocScratchBytes);
+    return kReduceScratchTooSmall;
+  }
+  FixedScratch fixed{nullptr, kNoAllocScratchBytes};
+  if (need > 0) {
+    fixed.ptr = noalloc_scratch_of_current_device(__func__);
+    if (!fixed.ptr) return kReduceScratchUnavailable;
+  }
+  // Every partial that the second kernel reads is written by the first kernel of the same call, so nothing in
+  // the array has to start at zero.
+  return launch_chan_reduce(__func__, dim0, dim1, dim2,
+                            MeanVarReduce{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)}, x, nullptr,
+                            stream, nullptr, &fixed);
 }
 
 ANODE_EXPORT void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,

@@ -207,6 +207,16 @@ void anode_gpu_quantize_u8_packed_f32(uint32_t len, float lo, float hi, const fl
 void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, uint32_t outer_dim, const float *scale, const float *shift, const uint8_t *x, float *y, ANODE_LAUNCH_TAIL);
 /* batch_mean and batch_var in one pass over x: mean[c], var[c] = biased variance + epsilon (composes with batch_norm). */
 void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, float *mean, float *var, ANODE_LAUNCH_TAIL);
+/* batch_mean_var for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (whose one-block-per-channel reductions need no
+ * workspace).  Same kernels, geometry and results as anode_gpu_batch_mean_var_3d1_packed_f32, but the partial sums
+ * go to a 4 MiB device array that is part of the library image (one copy per GPU, held until the process ends)
+ * instead of the per-stream buffer: the call makes no hipMalloc / hipFree and no allocating library call.  Returns
+ * 0, or non-zero with nothing enqueued: 1 = the shape needs more than 4 MiB of partial sums (2 * dim1 * tiles per
+ * channel doubles; use the entry point above), 2 = the array's device address could not be obtained.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two threads, two graphs replayed together)
+ * race; calls in stream order on one stream do not. */
+int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, float *mean, float *var, ANODE_LAUNCH_TAIL);
 /* batch_norm followed by positive_clip in one pass: t = (x-mean[c])*rsqrt(var[c]); y = t * float(t>0). */
 void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, const float *mean, const float *var, float *y, ANODE_LAUNCH_TAIL);
 /* batch_norm followed by the per-channel affine in one pass: y = fma((x-mean[c])*rsqrt(var[c]), gamma[c], beta[c]). */

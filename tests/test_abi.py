@@ -160,6 +160,10 @@ print("reserve", rc, take(), take())
 # [12544, 64, 256] needs partial sums: the reduction must give up, record the error and return
 lib.symbol("anode_gpu_batch_mean_3d1_packed_f32")(12544, 64, 256, None, None, ctypes.byref(cfg), None)
 print("mean", take(), take())
+# the entry point that never allocates refuses an oversized shape before it touches the device
+rc = lib.symbol("anode_gpu_batch_mean_var_3d1_packed_noalloc_f32")(1, 65536, 4096, 1e-5, None, None, None,
+                                                                   ctypes.byref(cfg), None)
+print("noalloc", rc, take())
 print("released", lib.symbol("anode_gpu_release_scratch")(None))
 print("alive")
 """
@@ -177,9 +181,11 @@ def test_scratch_allocation_failure_is_reported_not_fatal():
     assert rc != 0 and err == rc and again == 0          # reported once, then cleared
     err, again = (int(v) for v in out["mean"])
     assert err != 0 and again == 0
+    assert out["noalloc"] == ["1", "0"]                  # refused by size: not a HIP error
     assert out["released"] == ["0"] and "alive" in out
     assert "cannot allocate the reduction scratch" in r.stderr and "nothing was enqueued" in r.stderr
     assert "anode_gpu_batch_mean_3d1_packed_f32" in r.stderr
+    assert "more than the 4194304 bytes of the static scratch array" in r.stderr
 
 
 def test_scratch_size_query_bounds_the_plan():

@@ -1,0 +1,78 @@
+"""The entry point that allocates nothing: anode_gpu_batch_mean_var_3d1_packed_noalloc_f32 keeps its partial sums
+in a device array that is part of the library image.  Its output must equal that of the allocating entry point,
+anode_gpu_batch_mean_var_3d1_packed_f32, to the bit (same kernels, same tiling), also on a second call with a
+smaller input, which finds the first call's partial sums still in the array."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from anode_amd import gpu
+from anode_amd._lib import load
+from gpu_util import F32, assert_bit_exact, assert_close, call, dev, empty, host
+
+pytestmark = pytest.mark.gpu
+
+NOALLOC = "anode_gpu_batch_mean_var_3d1_packed_noalloc_f32"
+PLAIN = "anode_gpu_batch_mean_var_3d1_packed_f32"
+
+
+def _noalloc(S, C, N, eps, x, mean, var, stream=None):
+    lib = load()
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.symbol(NOALLOC)(S, C, N, eps, x.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                             ctypes.byref(gpu.DEFAULT_CONFIG), ctypes.c_void_p(stream))
+    assert gpu.take_last_error() == 0
+    return rc
+
+
+def _one(oracle, S, C, N, seed, offset=0):
+    print(f"noalloc case S={S} C={C} N={N} seed={seed} offset={offset}", flush=True)
+    g = np.random.default_rng(seed)
+    x = (2 + 3 * g.standard_normal(S * C * N)).astype(F32)
+    xd = dev(x, offset)
+    mean_a, var_a, mean_b, var_b = empty(C), empty(C), empty(C), empty(C)
+    assert _noalloc(S, C, N, 1e-5, xd, mean_a, var_a) == 0
+    call(PLAIN, S, C, N, 1e-5, xd, mean_b, var_b)
+    assert_bit_exact(host(mean_a), host(mean_b), f"mean [{S},{C},{N}]")
+    assert_bit_exact(host(var_a), host(var_b), f"var [{S},{C},{N}]")
+    m64, v64 = oracle.batch_mean_var(S, C, N, 1e-5, x)
+    assert_close(host(mean_a), m64, "mean vs fp64 oracle")
+    assert_close(host(var_a), v64, "var vs fp64 oracle")
+
+
+def test_two_calls_in_a_row_second_smaller(oracle):
+    # first call: many tiles per channel (chunk tiles); second: fewer and smaller partial lists in the same array,
+    # which still holds the first call's sums
+    _one(oracle, 12544, 16, 32, seed=1)
+    _one(oracle, 49, 40, 24, seed=2)
+    _one(oracle, 5000, 3, 5, seed=3, offset=1)   # element-aligned input
+    _one(oracle, 7, 5, 1, seed=4)                # one tile per channel: no partial sums at all
+
+
+def test_stream_order_keeps_calls_apart():
+    # back-to-back calls on one stream share the array; stream order is enough
+    S, C, N = 784, 16, 64
+    g = np.random.default_rng(7)
+    xs = [dev((k + g.standard_normal(S * C * N)).astype(F32)) for k in range(4)]
+    outs = [(empty(C), empty(C)) for _ in xs]
+    refs = [(empty(C), empty(C)) for _ in xs]
+    for x, (m, v) in zip(xs, outs):
+        assert _noalloc(S, C, N, 1e-5, x, m, v) == 0
+    for x, (m, v) in zip(xs, refs):
+        call(PLAIN, S, C, N, 1e-5, x, m, v)
+    for (m, v), (rm, rv) in zip(outs, refs):
+        assert_bit_exact(host(m), host(rm), "mean")
+        assert_bit_exact(host(v), host(rv), "var")
+
+
+def test_oversized_shape_is_refused():
+    # [1, 65536, 4096]: 32 partials for each of 65536 channels, two sums -> 32 MiB > 4 MiB; nothing may be written
+    S, C, N = 1, 65536, 4096
+    x = torch.zeros(8, device="cuda")  # never read
+    mean, var = empty(4), empty(4)
+    assert _noalloc(S, C, N, 1e-5, x, mean, var) == 1
+    torch.cuda.synchronize()
+    assert np.all(np.isnan(host(mean))) and np.all(np.isnan(host(var)))
