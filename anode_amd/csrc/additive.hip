@@ -495,7 +495,8 @@ ANODE_EXPORT int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, 
                                                                  CUstream_st *stream) {
   // Sizes are checked before anything touches the device, so that a refusal has no side effect.
   const bool ptrs_aligned = aligned16(x);
-  const ReducePlan pl = plan_chan_reduce(dim0, dim1, dim2, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
+  const ReducePlan pl = plan_chan_reduce(dim0, dim1, dim2, ptrs_aligned, uint32_t(tuning().reduce_wg_target),
+                                         MeanVarReduce::NIN);
   const size_t need = chan_reduce_scratch_bytes(pl, MeanVarReduce::NACC);
   if (need > kNoAllocScratchBytes) {
     std::fprintf(stderr,

@@ -28,18 +28,24 @@
 
 namespace anode {
 
-constexpr uint32_t kTilePos = 4096;   // positions of a "whole" tile: 32 KiB of fp64 in LDS
-// LDS slot of tile position p.  A thread owns four consecutive positions; storing them in four planes lets the 64
-// lanes of a wave write consecutive doubles, and the plane pitch (1024 + 16 doubles, i.e. 32 banks off a multiple of
-// 64) keeps the channel-wise read of consecutive positions at two lanes per bank pair, the minimum for 8-byte
-// accesses.  (Stored in position order, every eighth lane hit the same banks: 45 % of the LDS cycles were conflicts.)
-constexpr uint32_t kTilePlane = kTilePos / 4 + 16;
-__host__ __device__ inline uint32_t tile_slot(uint32_t p) { return (p & 3u) * kTilePlane + (p >> 2); }
+// Positions of a "whole" tile: 1024, 2048 or 4096 (8 to 32 KiB of fp64 in LDS), the smallest that holds the tile.
+// A narrow tile over more samples reads the same bytes as a wide one over fewer, but its epilogue (per-position sums
+// through LDS) is a quarter of the work, it leaves room for four times as many workgroups per compute unit and a
+// thread carries 4 instead of 16 running sums per statistic.
+constexpr uint32_t kTilePos = 4096;     // the widest tile: bounds S of the whole-channel form
+constexpr uint32_t kTilePosMin = 1024;  // the narrowest: one 16-byte group per thread
+// LDS slot of tile position p in a tile of P positions.  A thread owns four consecutive positions; storing them in
+// four planes lets the 64 lanes of a wave write consecutive doubles, and the plane pitch (P/4 + 16 doubles, i.e. 32
+// banks off a multiple of 64) keeps the channel-wise read of consecutive positions at two lanes per bank pair, the
+// minimum for 8-byte accesses.  (Stored in position order, every eighth lane hit the same banks: 45 % of the LDS
+// cycles were conflicts.)
+template <uint32_t P>
+__host__ __device__ inline uint32_t tile_slot(uint32_t p) { return (p & 3u) * (P / 4 + 16) + (p >> 2); }
 constexpr uint32_t kMaxTileChans = 256;
 
 struct ReducePlan {
   uint32_t S, C, N;
-  uint32_t whole;     // 1: whole-channel tiles, 0: chunk tiles
+  uint32_t whole;     // 0: chunk tiles, 1: wide whole-channel tiles, 2: lane tiles
   uint32_t CB;        // channels per tile (whole)
   uint32_t SB;        // positions per tile (chunk)
   uint32_t n_ctiles;  // whole: ceil(C / CB); chunk: C
@@ -49,12 +55,14 @@ struct ReducePlan {
   uint32_t ppc;       // partials per channel = n_stiles * n_ntiles
   uint32_t vec;       // 1: 16-byte accesses are legal for this geometry
   uint32_t grid;      // n_ctiles * n_stiles * n_ntiles
+  uint32_t P;         // wide tiles: positions per tile (1024, 2048 or 4096); otherwise 0
+  uint32_t J;         // lane tiles: samples that the lanes of a workgroup take side by side; otherwise 0
 };
 
 // Host-side tiling decision; `ptrs_aligned` says whether every element array
-// is 16-byte aligned.  Exposed (anode_gpu_plan_reduce) so that it can be
+// is 16-byte aligned, `nin` how many element arrays the reduction reads.  Exposed (anode_gpu_plan_reduce) so that it can be
 // checked without a device.
-ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target);
+ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target, int nin);
 
 #if defined(__HIPCC__)
 
@@ -149,16 +157,19 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
   }
 }
 
-template <typename Op, typename V, int NT>
+template <typename Op, typename V, int NT, uint32_t P>
 __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl, FastDiv div_s, Op op,
                                                                    const float *__restrict__ a,
                                                                    const float *__restrict__ b,
                                                                    const float *__restrict__ c3,
                                                                    double *__restrict__ part) {
   constexpr int W = VecLanes<V>::n;
-  constexpr int G = 16 / W;                       // position groups owned by a thread
-  constexpr int STAGES = (Op::NIN >= 2) ? 1 : 2;  // samples loaded before any is consumed
-  __shared__ double lds[4 * kTilePlane];
+  constexpr int G = int(P / kBlock) / W;  // position groups owned by a thread
+  // samples loaded before any is consumed: about eight 16-byte (or thirty-two 4-byte) loads in flight per thread
+  constexpr int LOADS = G * Op::NIN;
+  constexpr int TARGET = (W == 1) ? 32 : 8;
+  constexpr int STAGES = LOADS >= TARGET ? 1 : TARGET / LOADS;
+  __shared__ double lds[P + 64];
 
   const uint32_t ct = blockIdx.x % pl.n_ctiles;
   const uint32_t nt = blockIdx.x / pl.n_ctiles;
@@ -237,7 +248,7 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
       if (valid[i]) {
 #pragma unroll
         for (int k = 0; k < W; ++k) {
-          lds[tile_slot((threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W) + uint32_t(k))] =
+          lds[tile_slot<P>((threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W) + uint32_t(k))] =
               q == 0 ? acc0[i][k] : (q == 1 ? acc1[i][k] : acc2[i][k]);
         }
       }
@@ -246,7 +257,126 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
     double s = 0.0;
     if (cl < cb) {
       const uint32_t first = cl * pl.S;
-      for (uint32_t ss = jj; ss < pl.S; ss += tpc) s += lds[tile_slot(first + ss)];
+      for (uint32_t ss = jj; ss < pl.S; ss += tpc) s += lds[tile_slot<P>(first + ss)];
+    }
+    res[q] = group_sum(s, int(tpc));
+  }
+  if (cl < cb && jj == 0) {
+    const uint32_t c = c0 + cl;
+    if (pl.ppc == 1) {
+      op.finalize(c, res[0], res[1], res[2]);
+    } else {
+      const size_t plane = size_t(pl.C) * pl.ppc;
+      const size_t slot = size_t(c) * pl.ppc + nt;
+      part[slot] = res[0];
+      if (Op::NACC >= 2) part[plane + slot] = res[1];
+      if (Op::NACC >= 3) part[2 * plane + slot] = res[2];
+    }
+  }
+}
+
+// "Lane" tiles, for short channels (CB*S positions fit the lanes of one workgroup, 16 bytes per lane): lane t takes
+// group t % GPS of sample slot t / GPS, so J = 256 / GPS samples are read side by side and a thread always meets the
+// same positions, hence the same channels.  The tile runs over NB samples in steps of J (often all N: then a channel
+// has a single partial, nothing goes through the scratch buffer and there is no second kernel).  At the end the
+// per-position sums of all J slots meet in LDS and are folded to channels in a fixed order.
+template <typename Op, typename V, int NT>
+__global__ __launch_bounds__(kBlock) void chan_reduce_lanes_kernel(ReducePlan pl, FastDiv div_s, FastDiv div_g, Op op,
+                                                                   const float *__restrict__ a,
+                                                                   const float *__restrict__ b,
+                                                                   const float *__restrict__ c3,
+                                                                   double *__restrict__ part) {
+  constexpr int W = VecLanes<V>::n;
+  // samples per batch: all loads of a batch are requested before the first is consumed
+  // (4, 8 or 16 loads per batch and input measure the same at [49, 2048, 256]: 21.4, 21.6, 22.4 us)
+  constexpr int STAGES = Op::NIN == 1 ? 8 : (Op::NIN == 2 ? 4 : 2);
+  constexpr uint32_t P = 1024;  // LDS layout of tile_slot: kBlock threads x up to 4 positions
+  __shared__ double lds[P + 64];
+
+  const uint32_t ct = blockIdx.x % pl.n_ctiles;
+  const uint32_t nt = blockIdx.x / pl.n_ctiles;
+  const uint32_t c0 = ct * pl.CB;
+  const uint32_t cb = min(pl.CB, pl.C - c0);
+  const uint32_t gps_full = div_g.d;                   // groups per sample of a full tile: the lane pitch of a slot
+  const uint32_t gps = (cb * pl.S) / uint32_t(W);      // groups per sample of this tile
+  const uint32_t J = pl.J;
+  const uint32_t n0 = nt * pl.NB;
+  const uint32_t n1 = min(pl.N, n0 + pl.NB);
+  const size_t CS = size_t(pl.C) * pl.S;
+  uint32_t j, g;
+  div_g.divmod(threadIdx.x, j, g);
+  const bool active = j < J && g < gps;
+
+  double acc0[W], acc1[W], acc2[W];
+  typename Op::Param prm[W];
+#pragma unroll
+  for (int k = 0; k < W; ++k) {
+    acc0[k] = acc1[k] = acc2[k] = 0.0;
+    const uint32_t pos = active ? g * uint32_t(W) + uint32_t(k) : 0u;  // idle lanes read channel c0's parameters
+    prm[k] = op.load(c0 + div_s.div(pos));
+  }
+
+  if (active) {
+    const size_t off = size_t(c0) * pl.S + size_t(g) * W;
+    const uint64_t step = uint64_t(J) * uint32_t(STAGES);
+    auto request = [&](uint64_t n, V(&va)[STAGES], V(&vb)[STAGES], V(&vc)[STAGES]) {
+#pragma unroll
+      for (int sg = 0; sg < STAGES; ++sg) {
+        const uint64_t nn = n + uint64_t(sg) * J;
+        if (nn < n1) {
+          const size_t at = size_t(nn) * CS + off;
+          va[sg] = load_stream<NT>(reinterpret_cast<const V *>(a + at));
+          if (Op::NIN >= 2) vb[sg] = load_stream<NT>(reinterpret_cast<const V *>(b + at));
+          if (Op::NIN >= 3) vc[sg] = load_stream<NT>(reinterpret_cast<const V *>(c3 + at));
+        }
+      }
+    };
+    auto consume = [&](uint64_t n, const V(&va)[STAGES], const V(&vb)[STAGES], const V(&vc)[STAGES]) {
+#pragma unroll
+      for (int sg = 0; sg < STAGES; ++sg) {
+        const uint64_t nn = n + uint64_t(sg) * J;
+        if (nn < n1) {
+#pragma unroll
+          for (int k = 0; k < W; ++k) {
+            chan_reduce_term(op, prm[k], lane_get<V>(va[sg], k), (Op::NIN >= 2) ? lane_get<V>(vb[sg], k) : 0.0f,
+                             (Op::NIN >= 3) ? lane_get<V>(vc[sg], k) : 0.0f, acc0[k], acc1[k], acc2[k]);
+          }
+        }
+      }
+    };
+    // One batch at a time: requesting the next batch before the current one is consumed (twice the loads in
+    // flight) measured 31 us against 21.6 us for batch_mean at [49, 2048, 256] read from HBM.
+    V va[STAGES], vb[STAGES], vc[STAGES];
+    for (uint64_t n = uint64_t(n0) + j; n < n1; n += step) {
+      request(n, va, vb, vc);
+      consume(n, va, vb, vc);
+    }
+  }
+
+  // fold (slot, position) to channels: tpc consecutive lanes share one channel and walk its J*S sums, slot by slot
+  uint32_t tpc = 64;
+  while (tpc > 1 && tpc * cb > uint32_t(kBlock)) tpc >>= 1;
+  const uint32_t cl = threadIdx.x / tpc;
+  const uint32_t jj = threadIdx.x % tpc;
+  const uint32_t per_chan = J * pl.S;
+  double res[3] = {0.0, 0.0, 0.0};
+#pragma unroll
+  for (int q = 0; q < Op::NACC; ++q) {
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int k = 0; k < W; ++k) {
+        lds[tile_slot<P>(threadIdx.x * uint32_t(W) + uint32_t(k))] = q == 0 ? acc0[k] : (q == 1 ? acc1[k] : acc2[k]);
+      }
+    }
+    __syncthreads();
+    double s = 0.0;
+    if (cl < cb) {
+      for (uint32_t e = jj; e < per_chan; e += tpc) {
+        uint32_t slot, ss;
+        div_s.divmod(e, slot, ss);
+        s += lds[tile_slot<P>(slot * gps_full * uint32_t(W) + cl * pl.S + ss)];
+      }
     }
     res[q] = group_sum(s, int(tpc));
   }
@@ -347,7 +477,7 @@ int launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, O
     return kReduceOk;
   }
   const bool ptrs_aligned = aligned16(a) && (Op::NIN < 2 || aligned16(b)) && (Op::NIN < 3 || aligned16(c));
-  const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target));
+  const ReducePlan pl = plan_chan_reduce(S, C, N, ptrs_aligned, uint32_t(tuning().reduce_wg_target), Op::NIN);
   if (Op::NIN < 2) b = a;
   if (Op::NIN < 3) c = a;
   const int nt = stream_policy(size_t(len) * sizeof(float), tuning().reduce_nontemporal);
@@ -365,16 +495,38 @@ int launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, O
       part = static_cast<double *>(lease.ptr);
     }
   }
-  if (pl.whole) {
+  if (pl.whole == 2) {
     const FastDiv div_s(S);
+    const FastDiv div_g(uint32_t((uint64_t(pl.CB) * S + (pl.vec ? 3 : 0)) / (pl.vec ? 4 : 1)));
     if (pl.vec) {
       if (nt) {
-        chan_reduce_whole_kernel<Op, f32x4, kNtLoad><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+        chan_reduce_lanes_kernel<Op, f32x4, kNtLoad><<<pl.grid, kBlock, 0, s>>>(pl, div_s, div_g, op, a, b, c, part);
       } else {
-        chan_reduce_whole_kernel<Op, f32x4, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+        chan_reduce_lanes_kernel<Op, f32x4, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, div_g, op, a, b, c, part);
       }
     } else {
-      chan_reduce_whole_kernel<Op, float, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+      chan_reduce_lanes_kernel<Op, float, 0><<<pl.grid, kBlock, 0, s>>>(pl, div_s, div_g, op, a, b, c, part);
+    }
+  } else if (pl.whole) {
+    const FastDiv div_s(S);
+    auto launch_whole = [&](auto tile_positions) {
+      constexpr uint32_t P = decltype(tile_positions)::value;
+      if (pl.vec) {
+        if (nt) {
+          chan_reduce_whole_kernel<Op, f32x4, kNtLoad, P><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+        } else {
+          chan_reduce_whole_kernel<Op, f32x4, 0, P><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+        }
+      } else {
+        chan_reduce_whole_kernel<Op, float, 0, P><<<pl.grid, kBlock, 0, s>>>(pl, div_s, op, a, b, c, part);
+      }
+    };
+    if (pl.P == 1024) {
+      launch_whole(std::integral_constant<uint32_t, 1024>{});
+    } else if (pl.P == 2048) {
+      launch_whole(std::integral_constant<uint32_t, 2048>{});
+    } else {
+      launch_whole(std::integral_constant<uint32_t, 4096>{});
     }
   } else {
     if (pl.vec) {

@@ -196,6 +196,11 @@ struct Tuning {
   Knob nt_min_bytes;       // arrays smaller than this keep the default cache policy (they fit the last-level cache)
   Knob reduce_min_tile;    // fewest elements a reduction tile reads (bounds the share of the per-tile epilogue)
   Knob nt_store_min_bytes; // arrays of at least this size are written with streaming stores (never above nt_min_bytes)
+  Knob reduce_tile_pos;    // 0: the reductions choose their tile width; 1024, 2048, 4096: forced where S allows
+  Knob reduce_lanes;             // 1: short channels (S <= 1024) use lane tiles (samples side by side in a workgroup)
+  Knob reduce_single_pass_grid;  // lane tiles: with at least this many channel groups a tile takes all samples
+  Knob reduce_lanes_max_ctiles;  // lane tiles: most channel groups (bounds the grid for very many channels)
+  Knob reduce_lanes_min_run;     // lane tiles: fewest contiguous floats a tile reads per sample
 };
 
 // The streaming mask to use for an array of `bytes` bytes: the load bit of `mask` from nt_min_bytes on, the store

@@ -35,7 +35,12 @@ Tuning g_tuning = {
     /*nt_min_bytes=*/{{192 << 20}},
     /*reduce_min_tile=*/{{16384}},
     /*nt_store_min_bytes=*/{{16 << 20}},
-};
+    /*reduce_tile_pos=*/{{0}},
+    /*reduce_lanes=*/{{1}},
+    /*reduce_single_pass_grid=*/{{256}},
+    /*reduce_lanes_max_ctiles=*/{{2048}},
+    /*reduce_lanes_min_run=*/{{128}},
+    };
 
 }  // namespace
 
@@ -123,7 +128,7 @@ uint32_t gcd_u32(uint32_t a, uint32_t b) {
 }
 }  // namespace
 
-ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target) {
+ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target, int nin) {
   ReducePlan p{};
   p.S = S;
   p.C = C;
@@ -155,29 +160,112 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
       p.NB = uint32_t(nb);
     }
   } else {
-    p.whole = 1;
     p.SB = S;
     p.n_stiles = 1;
-    uint32_t cb = kTilePos / S;
-    if (cb > kMaxTileChans) cb = kMaxTileChans;
-    if (cb > C) cb = C;
     bool vec = ptrs_aligned && (uint64_t(C) * S) % 4 == 0;
-    if (vec && cb != C) {
-      // every tile must start on a 16-byte boundary: CB*S a multiple of 4
-      const uint32_t unit = 4 / gcd_u32(S, 4);
-      if (cb >= unit) {
-        cb -= cb % unit;
-      } else {
-        vec = false;
+    // a tile that is not the whole channel axis must start on a 16-byte boundary: CB*S a multiple of 4
+    const uint32_t unit = 4 / gcd_u32(S, 4);
+    const uint32_t lane_cap = kBlock * (vec ? 4u : 1u);  // positions that one pass of a workgroup's lanes covers
+    bool lanes = g_tuning.reduce_lanes > 0 && S <= lane_cap && (!vec || C <= unit || unit * S <= lane_cap);
+    if (lanes) {
+      // "lane" tiles: few channels, all (or many) samples, several samples side by side in the workgroup
+      uint32_t cb_max = lane_cap / S;
+      if (cb_max > kMaxTileChans) cb_max = kMaxTileChans;
+      if (cb_max >= C) {
+        cb_max = C;
+      } else if (vec) {
+        cb_max -= cb_max % unit;
       }
+      // (with two or more input arrays twice the run: measured 34.5 us against 37.0 us for batch_norm_bwd_var at
+      // [49, 2048, 256], while one-input reductions lose 2 us with the longer run)
+      const uint32_t run = (g_tuning.reduce_lanes_min_run > 0 ? uint32_t(g_tuning.reduce_lanes_min_run) : 1u) *
+                           (nin >= 2 ? 2u : 1u);
+      const uint32_t max_ctiles = g_tuning.reduce_lanes_max_ctiles > 0 ? uint32_t(g_tuning.reduce_lanes_max_ctiles) : 1u;
+      uint32_t cb = ceil_div_u32(run, S);                 // a sample's run of the tile is at least `run` floats long
+      const uint32_t fit = ceil_div_u32(C, max_ctiles);   // and the grid stays bounded
+      if (cb < fit) cb = fit;
+      if (vec) cb = ceil_div_u32(cb, unit) * unit;
+      if (cb > cb_max) cb = cb_max;
+      {
+        // among the legal widths from there on, the one that keeps most lanes busy (J slots of gps lanes each)
+        const uint32_t step = (vec && cb_max != C) ? unit : 1u;
+        const uint32_t w = vec ? 4u : 1u;
+        uint32_t best = cb, best_busy = 0;
+        for (uint32_t k = cb; k <= cb_max && k < cb + 64 * step; k += step) {
+          if (vec && k != C && k % unit != 0) continue;
+          const uint32_t gps_k = ceil_div_u32(uint64_t(k) * S, w);
+          const uint32_t busy = (kBlock / gps_k) * gps_k;
+          if (busy > best_busy && ceil_div_u32(C, k) * 2 >= ceil_div_u32(C, cb)) {
+            best = k;
+            best_busy = busy;
+          }
+        }
+        cb = best;
+      }
+      p.whole = 2;
+      p.CB = cb;
+      p.vec = vec ? 1 : 0;
+      p.n_ctiles = ceil_div_u32(C, cb);
+      const uint32_t gps = ceil_div_u32(uint64_t(cb) * S, vec ? 4u : 1u);  // 16-byte (or 4-byte) groups per sample
+      p.J = kBlock / gps;
+      if (p.n_ctiles >= uint32_t(g_tuning.reduce_single_pass_grid)) {
+        p.NB = N;  // one tile per channel group: no partial sums, no second kernel
+      } else {
+        uint64_t nb = per_tile / (uint64_t(cb) * S);
+        if (nb < p.J) nb = p.J;
+        if (nb > N) nb = N;
+        p.NB = uint32_t(nb);
+      }
+    } else {
+      p.whole = 1;
+      // channels of a tile of P positions, and whether it keeps 16-byte accesses (CB*S a multiple of 4)
+      auto fit = [&](uint32_t P, uint32_t &cb_out) {
+        uint32_t k = P / S;
+        if (k > kMaxTileChans) k = kMaxTileChans;
+        if (k > C) k = C;
+        bool v = vec && k > 0;
+        if (v && k != C) {
+          if (k >= unit) {
+            k -= k % unit;
+          } else {
+            v = false;
+          }
+        }
+        cb_out = k;
+        return v;
+      };
+      // the narrowest tile width that keeps 16-byte accesses (where any does) and wastes at most an eighth of
+      // its positions; failing that, the widest
+      uint32_t P = kTilePos, cb = 0;
+      bool any_vec = false;
+      for (uint32_t q = kTilePosMin; q <= kTilePos; q <<= 1) {
+        uint32_t k;
+        any_vec = any_vec || (q >= S && fit(q, k));
+      }
+      for (uint32_t q = kTilePosMin; q <= kTilePos; q <<= 1) {
+        uint32_t k;
+        if (q < S) continue;
+        const bool v = fit(q, k);
+        if (v == any_vec && uint64_t(k) * S * 8 >= uint64_t(q) * 7) {
+          P = q;
+          break;
+        }
+      }
+      if (g_tuning.reduce_tile_pos >= int(kTilePosMin) && uint32_t(g_tuning.reduce_tile_pos) >= S) {
+        P = uint32_t(g_tuning.reduce_tile_pos) >= kTilePos ? kTilePos : (g_tuning.reduce_tile_pos >= 2048 ? 2048u : 1024u);
+      }
+      vec = fit(P, cb);
+      // few channels: a narrower tile holds them just as well
+      while (P > kTilePosMin && uint64_t(cb) * S <= P / 2) P >>= 1;
+      p.P = P;
+      p.CB = cb;
+      p.vec = vec ? 1 : 0;
+      p.n_ctiles = ceil_div_u32(C, cb);
+      uint64_t nb = per_tile / (uint64_t(cb) * S);
+      if (nb < 1) nb = 1;
+      if (nb > N) nb = N;
+      p.NB = uint32_t(nb);
     }
-    p.CB = cb;
-    p.vec = vec ? 1 : 0;
-    p.n_ctiles = ceil_div_u32(C, cb);
-    uint64_t nb = per_tile / (uint64_t(cb) * S);
-    if (nb < 1) nb = 1;
-    if (nb > N) nb = N;
-    p.NB = uint32_t(nb);
   }
   p.n_ntiles = ceil_div_u32(N, p.NB);
   p.NB = ceil_div_u32(N, p.n_ntiles);  // balance the samples over the tiles
@@ -234,9 +322,14 @@ ANODE_EXPORT uint32_t anode_gpu_reference_symbol_count(void) { return 46; }
 // Upper bound of the partial-sum bytes a reduction over [S, C, N] needs: three sums, either alignment.
 ANODE_EXPORT size_t anode_gpu_reduce_scratch_bytes(uint32_t S, uint32_t C, uint32_t N) {
   const uint32_t target = uint32_t(anode::tuning().reduce_wg_target);
-  const size_t a = anode::chan_reduce_scratch_bytes(anode::plan_chan_reduce(S, C, N, true, target), 3);
-  const size_t b = anode::chan_reduce_scratch_bytes(anode::plan_chan_reduce(S, C, N, false, target), 3);
-  return a > b ? a : b;
+  size_t most = 0;
+  for (int nin = 1; nin <= 2; ++nin) {
+    for (int aligned = 0; aligned <= 1; ++aligned) {
+      const size_t b = anode::chan_reduce_scratch_bytes(anode::plan_chan_reduce(S, C, N, aligned != 0, target, nin), 3);
+      if (b > most) most = b;
+    }
+  }
+  return most;
 }
 
 // Makes sure that the reduction entry points find at least `bytes` of partial-sum scratch for `stream` on the
@@ -265,12 +358,14 @@ ANODE_EXPORT int anode_gpu_release_scratch(CUstream_st *stream) {
 }
 
 // Host-only view of the reduction tiling for a [S, C, N] array, as 12 words:
-// whole, CB, SB, n_ctiles, n_stiles, NB, n_ntiles, ppc, vec, grid, 0, 0.
+// whole, CB, SB, n_ctiles, n_stiles, NB, n_ntiles, ppc, vec, grid, P, J.
 ANODE_EXPORT void anode_gpu_plan_reduce(uint32_t S, uint32_t C, uint32_t N, int ptrs_aligned,
                                         uint32_t *out12) {
-  const anode::ReducePlan p =
-      anode::plan_chan_reduce(S, C, N, ptrs_aligned != 0, uint32_t(anode::tuning().reduce_wg_target));
-  const uint32_t v[12] = {p.whole, p.CB, p.SB, p.n_ctiles, p.n_stiles, p.NB, p.n_ntiles, p.ppc, p.vec, p.grid, 0, 0};
+  // bit 1 of ptrs_aligned set: the plan of a reduction with two or more input arrays
+  const anode::ReducePlan p = anode::plan_chan_reduce(S, C, N, (ptrs_aligned & 1) != 0,
+                                                      uint32_t(anode::tuning().reduce_wg_target),
+                                                      (ptrs_aligned & 2) ? 2 : 1);
+  const uint32_t v[12] = {p.whole, p.CB, p.SB, p.n_ctiles, p.n_stiles, p.NB, p.n_ntiles, p.ppc, p.vec, p.grid, p.P, p.J};
   std::memcpy(out12, v, sizeof(v));
 }
 
@@ -280,7 +375,8 @@ ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return a
 
 // Test and measurement hook (not declared in the public header).  Knobs: 0 flat_wg_per_cu, 2 reduce_wg_target,
 // 3 nontemporal (0, 1 or 3: streaming loads without streaming stores is not a policy the maps are built for),
-// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes.  Returns the previous value; a
+// 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes, 8 reduce_tile_pos,
+// 9 reduce_lanes, 10 reduce_single_pass_grid, 11 reduce_lanes_max_ctiles, 12 reduce_lanes_min_run.  Returns the previous value; a
 // negative value only reads.  Returns -1, and changes nothing, for an unknown knob or a value the knob does not take.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
   anode::Tuning &t = anode::tuning();
@@ -293,6 +389,11 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 5: slot = &t.nt_min_bytes; break;
     case 6: slot = &t.reduce_min_tile; break;
     case 7: slot = &t.nt_store_min_bytes; break;
+    case 8: slot = &t.reduce_tile_pos; break;
+    case 9: slot = &t.reduce_lanes; break;
+    case 10: slot = &t.reduce_single_pass_grid; break;
+    case 11: slot = &t.reduce_lanes_max_ctiles; break;
+    case 12: slot = &t.reduce_lanes_min_run; break;
     default: return -1;
   }
   if (knob == 3 && value >= 0 && value != 0 && value != 1 && value != 3) return -1;

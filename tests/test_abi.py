@@ -161,6 +161,8 @@ print("reserve", rc, take(), take())
 lib.symbol("anode_gpu_batch_mean_3d1_packed_f32")(12544, 64, 256, None, None, ctypes.byref(cfg), None)
 print("mean", take(), take())
 # the entry point that never allocates refuses an oversized shape before it touches the device
+# (tuning knob 9 = 0: without lane tiles this shape is cut into 32 sample tiles per channel group)
+lib.cdll.anode_gpu_set_tuning(9, 0)
 rc = lib.symbol("anode_gpu_batch_mean_var_3d1_packed_noalloc_f32")(1, 65536, 4096, 1e-5, None, None, None,
                                                                    ctypes.byref(cfg), None)
 print("noalloc", rc, take())
@@ -230,34 +232,80 @@ def test_exact_division_helper_matches_integer_division():
 def _plan(S, C, N, aligned=True):
     out = (ctypes.c_uint32 * 12)()
     _lib.load().cdll.anode_gpu_plan_reduce(S, C, N, int(aligned), out)
-    keys = ["whole", "CB", "SB", "n_ctiles", "n_stiles", "NB", "n_ntiles", "ppc", "vec", "grid"]
-    return dict(zip(keys, list(out)[:10]))
+    keys = ["whole", "CB", "SB", "n_ctiles", "n_stiles", "NB", "n_ntiles", "ppc", "vec", "grid", "P", "J"]
+    return dict(zip(keys, list(out)))
 
 
-@pytest.mark.parametrize("S,C,N", [
+PLAN_SHAPES = [
     (784, 16, 32), (12544, 64, 256), (49, 2048, 256), (2097152, 32, 2), (1, 1000, 64), (1, 1, 1), (3, 5, 7),
-    (4097, 3, 9), (4096, 1, 1), (50, 3, 2), (12321, 8, 4), (7, 300000, 2), (100000, 4, 1),
-])
+    (4097, 3, 9), (4096, 1, 1), (50, 3, 2), (12321, 8, 4), (7, 300000, 2), (100000, 4, 1), (1024, 3, 4), (1023, 7, 4),
+    (1025, 5, 3), (196, 512, 64), (300, 64, 32), (2, 3, 1000), (1, 65536, 4096), (255, 9, 2), (257, 9, 2),
+]
+
+
+def _check_plan(p, S, C, N, aligned):
+    assert p["grid"] == p["n_ctiles"] * p["n_stiles"] * p["n_ntiles"] >= 1
+    assert p["ppc"] == p["n_stiles"] * p["n_ntiles"]
+    assert (p["n_ntiles"] - 1) * p["NB"] < N <= p["n_ntiles"] * p["NB"]
+    if p["vec"]:
+        assert aligned
+    if p["whole"] == 2:    # lane tiles: CB*S positions fit the 256 lanes of a workgroup, 16 (or 4) bytes per lane
+        lanes = 4 if p["vec"] else 1
+        assert S <= 256 * lanes and 1 <= p["CB"] <= 256 and p["CB"] * S <= 256 * lanes
+        assert (p["n_ctiles"] - 1) * p["CB"] < C <= p["n_ctiles"] * p["CB"]
+        assert p["n_stiles"] == 1
+        groups = -(-p["CB"] * S // lanes)
+        assert p["J"] == 256 // groups >= 1
+        if p["vec"]:
+            assert (C * S) % 4 == 0 and (p["CB"] == C or (p["CB"] * S) % 4 == 0)
+    elif p["whole"] == 1:  # wide tiles
+        assert S <= 4096 and p["P"] in (1024, 2048, 4096) and p["CB"] * S <= p["P"] and 1 <= p["CB"] <= 256
+        assert (p["n_ctiles"] - 1) * p["CB"] < C <= p["n_ctiles"] * p["CB"]
+        assert p["n_stiles"] == 1
+        if p["vec"]:
+            assert (C * S) % 4 == 0
+            assert p["CB"] == C or (p["CB"] * S) % 4 == 0  # every tile starts on a 16-byte boundary
+    else:                  # chunk tiles
+        assert S > 4096 and p["n_ctiles"] == C
+        assert (p["n_stiles"] - 1) * p["SB"] < S <= p["n_stiles"] * p["SB"]
+        if p["vec"]:
+            assert S % 4 == 0 and (p["SB"] % 4 == 0 or p["n_stiles"] == 1)
+
+
+@pytest.mark.parametrize("S,C,N", PLAN_SHAPES)
 def test_reduction_tiling_covers_the_array_exactly_once(S, C, N):
     for aligned in (True, False):
         p = _plan(S, C, N, aligned)
-        assert p["grid"] == p["n_ctiles"] * p["n_stiles"] * p["n_ntiles"] >= 1
-        assert p["ppc"] == p["n_stiles"] * p["n_ntiles"]
-        assert (p["n_ntiles"] - 1) * p["NB"] < N <= p["n_ntiles"] * p["NB"]
-        if p["whole"]:
-            assert S <= 4096 and p["CB"] * S <= 4096 and 1 <= p["CB"] <= 256
-            assert (p["n_ctiles"] - 1) * p["CB"] < C <= p["n_ctiles"] * p["CB"]
-            assert p["n_stiles"] == 1
-            if p["vec"]:
-                assert aligned and (C * S) % 4 == 0
-                assert p["CB"] == C or (p["CB"] * S) % 4 == 0  # every tile starts on a 16-byte boundary
-        else:
-            assert S > 4096 and p["n_ctiles"] == C
-            assert (p["n_stiles"] - 1) * p["SB"] < S <= p["n_stiles"] * p["SB"]
-            if p["vec"]:
-                assert aligned and S % 4 == 0 and (p["SB"] % 4 == 0 or p["n_stiles"] == 1)
+        _check_plan(p, S, C, N, aligned)
         if not aligned:
             assert not p["vec"]
+
+
+def test_reduction_tiling_without_lane_tiles():
+    # tuning knob 9 = 0 switches lane tiles off: short channels then use the wide tiles (in a child process, so that
+    # the knob does not leak into other tests)
+    code = r"""
+import ctypes, json, sys
+sys.path.insert(0, %r)
+from anode_amd import _lib
+lib = _lib.load()
+lib.cdll.anode_gpu_set_tuning(9, 0)
+out = {}
+for d in %r:
+    for al in (1, 0):
+        buf = (ctypes.c_uint32 * 12)()
+        lib.cdll.anode_gpu_plan_reduce(*d, al, buf)
+        out["%%d,%%d,%%d,%%d" %% (*d, al)] = list(buf)
+print(json.dumps(out))
+""" % (_lib.REPO_ROOT, PLAN_SHAPES)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120, check=True)
+    import json
+    keys = ["whole", "CB", "SB", "n_ctiles", "n_stiles", "NB", "n_ntiles", "ppc", "vec", "grid", "P", "J"]
+    for k, v in json.loads(r.stdout).items():
+        S, C, N, al = (int(t) for t in k.split(","))
+        p = dict(zip(keys, v))
+        assert p["whole"] != 2
+        _check_plan(p, S, C, N, bool(al))
 
 
 def test_product_package_never_reaches_the_oracle():

@@ -69,10 +69,18 @@ def test_stream_order_keeps_calls_apart():
 
 
 def test_oversized_shape_is_refused():
-    # [1, 65536, 4096]: 32 partials for each of 65536 channels, two sums -> 32 MiB > 4 MiB; nothing may be written
+    # With lane tiles switched off (tuning knob 9), [1, 65536, 4096] is cut into 32 sample tiles: 32 partials for
+    # each of 65536 channels, two sums -> 32 MiB > 4 MiB.  The call must return 1 and enqueue nothing.  The buffers
+    # have their full size all the same: a call that were accepted would only compute, never touch foreign memory.
     S, C, N = 1, 65536, 4096
-    x = torch.zeros(8, device="cuda")  # never read
-    mean, var = empty(4), empty(4)
-    assert _noalloc(S, C, N, 1e-5, x, mean, var) == 1
+    x = torch.empty(S * C * N, device="cuda")
+    mean, var = empty(C), empty(C)
+    saved = gpu.set_tuning(9, 0)
+    try:
+        assert load().symbol("anode_gpu_reduce_scratch_bytes")(S, C, N) > (4 << 20)
+        rc = _noalloc(S, C, N, 1e-5, x, mean, var)
+    finally:
+        gpu.set_tuning(9, saved)
     torch.cuda.synchronize()
+    assert rc == 1
     assert np.all(np.isnan(host(mean))) and np.all(np.isnan(host(var)))
