@@ -431,12 +431,33 @@ template <> struct PixVec<f32x4> {
 __device__ inline uint32_t lane_get_u(uint32_t v, int) { return v; }
 __device__ inline uint32_t lane_get_u(u32x4 v, int k) { return v[k]; }
 
-__device__ inline float vmax(float a, float b) { return fmaxf(a, b); }
-__device__ inline f32x4 vmax(f32x4 a, f32x4 b) {
-  return f32x4{fmaxf(a.x, b.x), fmaxf(a.y, b.y), fmaxf(a.z, b.z), fmaxf(a.w, b.w)};
+// max(a, b) as the single hardware instruction: a NaN operand yields the other operand and a signalling NaN is
+// quieted, which is fmaxf(); the library call costs two more instructions per element to canonicalise its inputs.
+__device__ inline float max1(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
 }
-__device__ inline float vexp(float a) { return expf(a); }
-__device__ inline f32x4 vexp(f32x4 a) { return f32x4{expf(a.x), expf(a.y), expf(a.z), expf(a.w)}; }
+__device__ inline float vmax(float a, float b) { return max1(a, b); }
+__device__ inline f32x4 vmax(f32x4 a, f32x4 b) {
+  return f32x4{max1(a.x, b.x), max1(a.y, b.y), max1(a.z, b.z), max1(a.w, b.w)};
+}
+
+// exp(d) for d <= 0 (the difference to a row's maximum): 2^(d * log2 e) with the hardware exponential, corrected
+// for the rounding of the product, r = fma(d, log2 e, -t), by the factor 1 + r ln 2.  Seven instructions instead of
+// the sixteen of expf(), which the n-d kernels feel: 76 exponentials per thread made them 40 % VALU-busy.
+// Relative error <= 3e-7 (+ 2e-8 |d| from the rounding of log2 e) while the result is a normal number; below
+// 2^-126 the hardware exponential returns 0, far under any probability that is compared (sums start at exp(0) = 1).
+// d = -inf gives 0 (the residual, inf - inf, is clamped before use), NaN gives NaN.
+__device__ inline float exp_nonpos(float d) {
+  constexpr float kLog2e = 1.44269502f, kLn2 = 0.693147182f;
+  const float t = d * kLog2e;
+  const float r = __builtin_amdgcn_fmed3f(fmaf(d, kLog2e, -t), -1.0f, 1.0f);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return fmaf(e, r * kLn2, e);
+}
+__device__ inline float vexp(float a) { return exp_nonpos(a); }
+__device__ inline f32x4 vexp(f32x4 a) { return f32x4{exp_nonpos(a.x), exp_nonpos(a.y), exp_nonpos(a.z), exp_nonpos(a.w)}; }
 __device__ inline float vrcp(float a) { return 1.0f / a; }
 __device__ inline f32x4 vrcp(f32x4 a) { return f32x4{1.0f / a.x, 1.0f / a.y, 1.0f / a.z, 1.0f / a.w}; }
 
@@ -456,65 +477,94 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
   p = r * uint32_t(W);
 }
 
-// C <= CMAX: the pixel's classes stay in registers, x is read once.  The sum
-// of exponentials is formed class by class in index order; the normalisation
-// multiplies by one correctly rounded reciprocal per pixel.  With NLL the
-// label gather is fused: nll = -log(the stored probability of the label), NaN
-// when the label is out of range, exactly what the separate gather returns.
-template <int CMAX, typename V, bool NLL, int NT>
+__device__ inline float pair_swap(float v) { return __shfl_xor(v, 1, kWave); }
+__device__ inline f32x4 pair_swap(f32x4 v) {
+  return f32x4{__shfl_xor(v.x, 1, kWave), __shfl_xor(v.y, 1, kWave), __shfl_xor(v.z, 1, kWave), __shfl_xor(v.w, 1, kWave)};
+}
+
+// C <= CMAX: the pixel's classes stay in registers, x is read once.  SPLIT lanes (1 or 2) share a group of W
+// pixels: lane h of the pair holds classes h, h + SPLIT, ... and the pair's maxima and sums meet through one lane
+// exchange each.  Two lanes per group halve a thread's state (ten 16-byte loads in flight instead of nineteen at
+// C = 19) and measured 112 us against 120 us at [512K, 19, 8]; four or eight lanes are slower again (118, 122 us:
+// a load instruction then covers several short runs).  A lane adds its exponentials in class order, the pair's sums
+// are added last; the normalisation multiplies by one correctly rounded reciprocal per pixel.  With NLL the label
+// gather is fused: nll = -log(the stored probability of the label), NaN when the label is out of range, exactly
+// what the separate gather returns.
+template <int CMAX, typename V, bool NLL, int NT, int SPLIT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 const uint32_t *__restrict__ cat,
                                                                 float *__restrict__ nll) {
   constexpr int W = PixVec<V>::W;
+  constexpr int H = (CMAX + SPLIT - 1) / SPLIT;  // classes a lane holds
   typedef typename PixVec<V>::U U;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t total = uint64_t(pg.total_groups) * SPLIT;
+  for (uint64_t t = uint64_t(blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
+    // the lanes of a pair are neighbours (t even, t + 1), so they always run, and leave the loop, together
+    const uint32_t g = uint32_t(t / SPLIT), h = uint32_t(t % SPLIT);
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
-    V v[CMAX];
+    V v[H];
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+      const uint32_t k = uint32_t(i) * SPLIT + h;
+      if (k < pg.C) v[i] = load_stream<NT>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
+    }
+    const size_t pix = size_t(p) + size_t(pg.P) * n;
+    U lab;
+    if (NLL) lab = *reinterpret_cast<const U *>(cat + pix);
     V m = PixVec<V>::splat(kNegInf);
 #pragma unroll
-    for (int k = 0; k < CMAX; ++k) {
-      if (uint32_t(k) < pg.C) {
-        v[k] = load_stream<NT>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
-        m = vmax(m, v[k]);
-      }
+    for (int i = 0; i < H; ++i) {
+      if (uint32_t(i) * SPLIT + h < pg.C) m = vmax(m, v[i]);
     }
+    if (SPLIT == 2) m = vmax(m, pair_swap(m));
     V s = PixVec<V>::splat(0.0f);
 #pragma unroll
-    for (int k = 0; k < CMAX; ++k) {
-      if (uint32_t(k) < pg.C) {
-        v[k] = vexp(v[k] - m);
-        s += v[k];
+    for (int i = 0; i < H; ++i) {
+      if (uint32_t(i) * SPLIT + h < pg.C) {
+        v[i] = vexp(v[i] - m);
+        s += v[i];
       }
     }
+    if (SPLIT == 2) s += pair_swap(s);  // a + b == b + a: both lanes hold the same sum
     const V inv = vrcp(s);
-    U lab;
-    V picked = PixVec<V>::splat(0.0f);
-    if (NLL) lab = *reinterpret_cast<const U *>(cat + (size_t(p) + size_t(pg.P) * n));
 #pragma unroll
-    for (int k = 0; k < CMAX; ++k) {
-      if (uint32_t(k) < pg.C) {
-        const V pr = v[k] * inv;
-        store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), pr);
-        if (NLL) {
-#pragma unroll
-          for (int w = 0; w < W; ++w) {
-            if (lane_get_u(lab, w) == uint32_t(k)) lane_set<V>(picked, w, lane_get<V>(pr, w));
-          }
-        }
-      }
+    for (int i = 0; i < H; ++i) {
+      const uint32_t k = uint32_t(i) * SPLIT + h;
+      if (k < pg.C) store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), v[i] * inv);
     }
     if (NLL) {
-      V out;
+      // The label's exponential is picked out of the registers of the lane that holds it (a compare and a select
+      // per held class and pixel) and handed to lane 0 of the pair, which multiplies it by the reciprocal as the
+      // stored probability was.  (Reading the label's logit again instead, one 4-byte gather per pixel of a line
+      // the wave had just requested, took 169 us against 109 us without NLL at [512K, 19, 8].)
+      V pick = PixVec<V>::splat(0.0f);
 #pragma unroll
-      for (int w = 0; w < W; ++w) {
-        lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(lane_get<V>(picked, w))
-                                                      : (pg.ignore ? 0.0f : __builtin_nanf("")));
+      for (int i = 0; i < H; ++i) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          if (lane_get_u(lab, w) / uint32_t(SPLIT) == uint32_t(i)) lane_set<V>(pick, w, lane_get<V>(v[i], w));
+        }
       }
-      *reinterpret_cast<V *>(nll + (size_t(p) + size_t(pg.P) * n)) = out;
+      if (SPLIT == 2) {
+        const V other = pair_swap(pick);
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          if (lane_get_u(lab, w) % 2u != h) lane_set<V>(pick, w, lane_get<V>(other, w));
+        }
+      }
+      if (h == 0) {
+        V out;
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          const float pr = lane_get<V>(pick, w) * lane_get<V>(inv, w);
+          lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr) : (pg.ignore ? 0.0f : __builtin_nanf("")));
+        }
+        *reinterpret_cast<V *>(nll + pix) = out;
+      }
     }
   }
 }
@@ -627,24 +677,25 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore
 // one pixel group per thread: the hardware dispatcher walks the array in order
 uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
-// C <= 32 only
+// C <= 32 only.  The 16-byte form runs two lanes per pixel group.
 template <typename V, bool NLL, int NT>
 void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
                               float *nll, hipStream_t s) {
+  constexpr int SPLIT = PixVec<V>::W == 4 ? 2 : 1;
   const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
-  const uint32_t blocks = pixel_blocks(pg.total_groups);
+  const uint32_t blocks = stream_grid(uint64_t(pg.total_groups) * SPLIT, 1);
   if (C <= 4) {
-    softmax_nd_reg_kernel<4, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<4, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 8) {
-    softmax_nd_reg_kernel<8, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<8, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 16) {
-    softmax_nd_reg_kernel<16, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
-  } else if (C <= 20) {  // 19 / 20 classes are common label sets; four registers per class saved buy a wave of occupancy
-    softmax_nd_reg_kernel<20, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<16, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+  } else if (C <= 20) {  // 19 / 20 classes are common label sets
+    softmax_nd_reg_kernel<20, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else if (C <= 24) {
-    softmax_nd_reg_kernel<24, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<24, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   } else {
-    softmax_nd_reg_kernel<32, V, NLL, NT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<32, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
   }
 }
 
@@ -689,9 +740,9 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
     const uint32_t blocks = pixel_blocks(pg.total_groups);
     if (C <= 64) {
-      softmax_nd_reg_kernel<64, float, false, 0><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      softmax_nd_reg_kernel<64, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     } else {
-      softmax_nd_reg_kernel<128, float, false, 0><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      softmax_nd_reg_kernel<128, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     }
   } else if (vec) {
     launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);

@@ -168,3 +168,32 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
         call("anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32", P, C, N, dev(dy, offset), p_d,
              dev(lab, offset), dxa)
         assert_bit_exact(host(dxa), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, dx_in=old), "nd bwd acc vs fp32")
+
+
+@pytest.mark.parametrize("C", [3, 19, 40, 200])
+def test_softmax_nd_special_values(oracle, C):
+    # register-resident (C <= 32, C <= 128) and streaming (C > 128) kernels: -inf entries get probability 0, a NaN
+    # poisons its pixel only, a pixel of +-1e30 and one of large equal values do not overflow, widely spread logits
+    # keep their small probabilities to the relative bar
+    P, N = 8, 2
+    g = np.random.default_rng(C)
+    x = g.standard_normal((N, C, P)).astype(F32)
+    x[0, :, 0] = -np.inf
+    x[0, 1, 0] = 1.0
+    x[0, :, 1] = 5.0
+    x[0, 0, 1], x[0, 1, 1] = 1e30, -1e30
+    x[0, 2, 2] = np.nan
+    x[0, :, 3] = 88.0
+    x[0, :, 4] = np.linspace(-60, 8, C)
+    x[1, :, 5] = np.linspace(-20, 20, C)
+    x[1, :, 6] = -np.inf          # nothing but -inf: NaN, as exp(-inf - -inf) is
+    for offset in (0, 1):
+        y = empty(x.size, offset=offset)
+        call("anode_gpu_softmax_nd_packed_f32", P, C, N, dev(x, offset), y)
+        p = host(y).reshape(N, C, P)
+        want = oracle.softmax_nd(P, C, N, x.ravel(), f64=True).reshape(N, C, P)
+        assert_close(p, want, f"n-d special values C={C}", abs_floor=1e-30)
+        assert p[0, 1, 0] == 1.0 and np.all(np.delete(p[0, :, 0], 1) == 0)
+        assert np.all(np.isnan(p[0, :, 2])) and np.all(np.isnan(p[1, :, 6]))
+        assert not np.any(np.isnan(np.delete(p.reshape(N * C, P), [2], axis=1)[:C]))
+        assert np.all(p[0, :, 3] == p[0, 0, 3]) and abs(float(p[0, 0, 3]) * C - 1) < 1e-6
