@@ -58,6 +58,43 @@ __global__ __launch_bounds__(kBlock) void quantize_u8x4_kernel(uint32_t n_groups
   }
 }
 
+// 16-byte form on both sides: lane l of a wave loads the 16-byte groups j*64 + l (j = 0..3) of the wave's 256, packs
+// each to a dword, and the wave gathers the dwords through LDS so that each lane stores 16 consecutive bytes: four
+// 1 KiB loads and one 1 KiB store per wave, all contiguous.  One tile per workgroup, 4096 elements.
+__global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t n_groups, uint32_t tail, float lo,
+                                                                float scale, const float *__restrict__ x,
+                                                                uint8_t *__restrict__ y) {
+  __shared__ __align__(16) uint32_t lds[kBlock * 4];
+  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+  uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
+  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // first group = first output dword
+  f32x4 v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint64_t g = wave_first + uint32_t(j) * kWave + lane;
+    v[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (g < n_groups) v[j] = load_stream<kNtLoad>(&x4[g]);
+  }
+  uint32_t d[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    d[j] = quantize_one(v[j].x, lo, scale) | (quantize_one(v[j].y, lo, scale) << 8) |
+           (quantize_one(v[j].z, lo, scale) << 16) | (quantize_one(v[j].w, lo, scale) << 24);
+  }
+  const u32x4 out = wave_gather_dwords(d, lds + wave * (kWave * 4));
+  const uint64_t first = wave_first + uint64_t(lane) * 4u;  // this lane's first output dword
+  if (first + 3u < n_groups) {
+    *reinterpret_cast<u32x4 *>(y4 + first) = out;
+  } else {
+    for (uint32_t k = 0; k < 4u && first + k < n_groups; ++k) y4[first + k] = out[k];
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_groups * 4u + threadIdx.x;
+    y[i] = uint8_t(quantize_one(x[i], lo, scale));
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void quantize_u8_scalar_kernel(uint32_t len, float lo, float scale,
                                                                     const float *__restrict__ x,
                                                                     uint8_t *__restrict__ y) {
@@ -135,6 +172,61 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t 
   }
   if (blockIdx.x == 0 && threadIdx.x < tail) {
     const uint32_t i = n_groups * 4u + threadIdx.x;
+    const uint32_t q = div_s.div(i);
+    const uint32_t c = q - div_c.div(q) * C;
+    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
+  }
+}
+
+// The 16-byte form of the same: one 16-byte load of 16 codes per lane, the wave's dwords re-dealt through LDS (see
+// wave_deal_dwords), each lane converts the four dwords it is dealt.  One tile per workgroup, 4096 codes.
+template <int NT>
+__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t n_dwords, uint32_t tail,
+                                                                        FastDiv div_s, FastDiv div_c,
+                                                                        const float *__restrict__ scale,
+                                                                        const float *__restrict__ shift,
+                                                                        const uint8_t *__restrict__ x,
+                                                                        float *__restrict__ y) {
+  __shared__ __align__(16) uint32_t lds[kBlock * 4];
+  const u32x4 *x16 = reinterpret_cast<const u32x4 *>(x);
+  f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
+  const uint32_t S = div_s.d, C = div_c.d;
+  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const uint64_t g16 = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
+  const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (g16 * 4u + 3u < n_dwords) {
+    v = load_stream<kNtLoad>(&x16[g16]);
+  } else if (g16 * 4u < n_dwords) {
+    const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
+    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = x4[g16 * 4u + k];
+  }
+  uint32_t w[4];
+  wave_deal_dwords(v, lds + wave * (kWave * 4), w);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint64_t d = wave_first + uint32_t(j) * kWave + lane;
+    if (d < n_dwords) {
+      uint32_t q, sp;
+      div_s.divmod(uint32_t(d) * 4u, q, sp);
+      uint32_t c = q - div_c.div(q) * C;
+      float a = scale[c], b = shift[c];
+      f32x4 r;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        r[k] = fmaf(a, float((w[j] >> (8 * k)) & 0xffu), b);
+        if (k < 3 && ++sp == S) {
+          sp = 0;
+          c = (c + 1 == C) ? 0 : c + 1;
+          a = scale[c];
+          b = shift[c];
+        }
+      }
+      store_stream<NT>(&y4[d], r);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_dwords * 4u + threadIdx.x;
     const uint32_t q = div_s.div(i);
     const uint32_t c = q - div_c.div(q) * C;
     y[i] = fmaf(scale[c], float(x[i]), shift[c]);
@@ -348,7 +440,11 @@ void launch_quantize(const char *symbol, uint32_t len, float lo, float hi, const
   if (len == 0) return;
   const float scale = (hi - lo) / 255.0f;
   hipStream_t s = as_stream(stream);
-  if (aligned16(x) && aligned4(y)) {
+  if (aligned16(x) && aligned16(y)) {
+    const uint32_t groups = len / 4, tail = len % 4;
+    const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
+    quantize_u8x16_kernel<<<blocks ? blocks : 1, kBlock, 0, s>>>(groups, tail, lo, scale, x, y);
+  } else if (aligned16(x) && aligned4(y)) {
     const uint32_t groups = len / 4, tail = len % 4;
     const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
     quantize_u8x4_kernel<<<blocks ? blocks : 1, kBlock, 0, s>>>(groups, tail, lo, scale, x, y);
@@ -416,7 +512,14 @@ ANODE_EXPORT void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32
   if (len == 0) return;
   hipStream_t s = as_stream(stream);
   const FastDiv div_s(inner_dim), div_c(bcast_dim);
-  if (aligned4(x) && aligned16(y)) {
+  if (aligned16(x) && aligned16(y)) {
+    const uint32_t dwords = len / 4, tail = len % 4;
+    const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
+    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
+      bcast_dequantize_u8x16_kernel<decltype(policy)::value>
+          <<<blocks ? blocks : 1, kBlock, 0, s>>>(dwords, tail, div_s, div_c, scale, shift, x, y);
+    });
+  } else if (aligned4(x) && aligned16(y)) {
     const uint32_t groups = len / 4, tail = len % 4;
     with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
       bcast_dequantize_u8x4_kernel<decltype(policy)::value>

@@ -108,12 +108,36 @@ __device__ inline void store_stream(V *p, V v) {
     // `nt` together with device scope (`sc1`: the line is written through instead of lingering dirty in the XCD's
     // L2): measured 6.72 TB/s against 6.60 TB/s for `nt` alone on an 822 MB copy.  The builtin cannot express the
     // pair, hence the instruction itself; it is an ordinary vector store.
-    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(v) : "memory");
+    // The s_nop keeps the following instruction two wait states away: a VALU write to the data registers of a
+    // store of more than 8 bytes needs that distance, and the compiler, which inserts it after its own stores,
+    // does not look into inline assembly (seen as wrong values stored by a kernel that recomputed the registers
+    // for its next store right away).
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
   } else if constexpr ((NT & kNtStore) != 0) {
     __builtin_nontemporal_store(v, p);
   } else {
     *p = v;
   }
+}
+
+// Re-dealing a wave's dwords through LDS, for kernels whose narrow side would otherwise move 4 bytes per lane.
+// `wave_lds` is the wave's own 256 dwords (16-byte aligned).  Every thread of the workgroup must call (barriers).
+//   deal:   lane l holds dwords 4l..4l+3 (one 16-byte load); afterwards out[j] is dword j*64 + l, so that whatever
+//           is then computed from out[j] is stored contiguously across the wave;
+//   gather: the inverse: lane l holds dword j*64 + l in in[j]; the result is dwords 4l..4l+3 for one 16-byte store.
+__device__ inline void wave_deal_dwords(u32x4 v, uint32_t *wave_lds, uint32_t (&out)[4]) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  *reinterpret_cast<u32x4 *>(wave_lds + lane * 4u) = v;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) out[j] = wave_lds[uint32_t(j) * kWave + lane];
+}
+__device__ inline u32x4 wave_gather_dwords(const uint32_t (&in)[4], uint32_t *wave_lds) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) wave_lds[uint32_t(j) * kWave + lane] = in[j];
+  __syncthreads();
+  return *reinterpret_cast<const u32x4 *>(wave_lds + lane * 4u);
 }
 
 template <typename T>

@@ -185,6 +185,48 @@ __global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, u
   }
 }
 
+// 16-byte form: each lane loads 16 codes in one access, the wave re-deals the dwords through LDS, and each lane
+// converts the four dwords it is dealt, so that every load (1 KiB) and every store (four of 1 KiB) of the wave is
+// contiguous.  One tile per workgroup, 4096 codes.  Measured 34.7 us against 35.8 us for the dword form at
+// [256,3,224,224].
+template <int NT, typename Op>
+__global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t n_dwords, uint32_t tail, Op op,
+                                                             const uint8_t *__restrict__ x,
+                                                             typename Op::out_t *__restrict__ y) {
+  typedef typename Op::out4_t O4;
+  __shared__ __align__(16) uint32_t lds[kBlock * 4];
+  const u32x4 *x16 = reinterpret_cast<const u32x4 *>(x);
+  O4 *y4 = reinterpret_cast<O4 *>(y);
+  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const uint64_t g16 = uint64_t(blockIdx.x) * kBlock + threadIdx.x;  // this lane's group of 16 codes
+  const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // the wave's first dword
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (g16 * 4u + 3u < n_dwords) {
+    v = load_stream<NT>(&x16[g16]);
+  } else if (g16 * 4u < n_dwords) {  // the last, partial group of the array: dword by dword
+    const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
+    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = x4[g16 * 4u + k];
+  }
+  uint32_t w[4];
+  wave_deal_dwords(v, lds + wave * (kWave * 4), w);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint64_t d = wave_first + uint32_t(j) * kWave + lane;
+    if (d < n_dwords) {
+      O4 r;
+      r.x = op(w[j] & 0xffu);
+      r.y = op((w[j] >> 8) & 0xffu);
+      r.z = op((w[j] >> 16) & 0xffu);
+      r.w = op(w[j] >> 24);
+      store_stream<NT>(&y4[d], r);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail) {
+    const uint32_t i = n_dwords * 4u + threadIdx.x;
+    y[i] = op(uint32_t(x[i]));
+  }
+}
+
 template <typename Op>
 __global__ __launch_bounds__(kBlock) void widen_u8_scalar_kernel(uint32_t len, Op op,
                                                                  const uint8_t *__restrict__ x,
@@ -199,7 +241,15 @@ void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, 
   if (len == 0) return;
   const Tuning &t = tuning();
   hipStream_t s = as_stream(stream);
-  if (aligned4(x) && aligned16(y)) {
+  if (aligned16(x) && aligned16(y)) {
+    const uint32_t dwords = len / 4, tail = len % 4;
+    const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
+    // the policy looks at the output, which is four times the input
+    const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
+    with_stream_policy(nt, [&](auto policy) {
+      widen_u8x16_kernel<decltype(policy)::value, Op><<<blocks ? blocks : 1, kBlock, 0, s>>>(dwords, tail, op, x, y);
+    });
+  } else if (aligned4(x) && aligned16(y)) {
     const uint32_t groups = len / 4, tail = len % 4;
     // the store policy looks at the output, which is four times the input
     const int nt = stream_policy(size_t(len) * 4, t.nontemporal);

@@ -26,10 +26,29 @@ constexpr float kNegInf = -__builtin_huge_valf();
 // row softmax
 // ---------------------------------------------------------------------------
 
+// Optional fused label gather of the row kernels (cat == nullptr: none).  The thread that has just stored the
+// label's probability p also writes nll = -log(p), the value the separate gather would read back and compute; a
+// label >= K gives NaN (or 0 with `ignore`), written by the thread that holds class 0.
+struct RowNll {
+  const uint32_t *cat;
+  float *nll;
+  bool ignore;
+  __device__ bool on() const { return cat != nullptr; }
+  __device__ uint32_t label(uint64_t r) const { return cat[r]; }
+  // called by the thread that holds class k of row r, with the stored probability
+  __device__ void emit(uint64_t r, uint32_t K, uint32_t label, uint32_t k, float prob) const {
+    if (k == label) {
+      nll[r] = -logf(prob);
+    } else if (k == 0 && label >= K) {
+      nll[r] = ignore ? 0.0f : __builtin_nanf("");
+    }
+  }
+};
+
 // K <= 64.  G = lanes per row (power of two >= K), log2g its logarithm.
 __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K, uint32_t R, uint32_t log2g,
                                                                      const float *__restrict__ x,
-                                                                     float *__restrict__ y) {
+                                                                     float *__restrict__ y, RowNll nl) {
   const uint32_t G = 1u << log2g;
   const uint32_t rows_per_wave = uint32_t(kWave) >> log2g;
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -46,7 +65,11 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
     const float m = group_max(v, int(G));
     const float z = valid ? expf(v - m) : 0.0f;
     const float s = group_sum(z, int(G));
-    if (valid) y[idx] = z / s;
+    if (valid) {
+      const float pr = z / s;
+      y[idx] = pr;
+      if (nl.on()) nl.emit(r, K, nl.label(r), k, pr);
+    }
   }
 }
 
@@ -57,7 +80,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
 template <int KMAX, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, FastDiv div_k, int vec,
                                                                  const float *__restrict__ x,
-                                                                 float *__restrict__ y) {
+                                                                 float *__restrict__ y, RowNll nl) {
   extern __shared__ float tile[];  // kBlock * (K|1) floats
   const uint32_t pitch = K | 1u;
   for (uint64_t r0 = uint64_t(blockIdx.x) * kBlock; r0 < R; r0 += uint64_t(gridDim.x) * kBlock) {
@@ -108,6 +131,11 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
       for (int k = 0; k < KMAX; ++k) {
         if (uint32_t(k) < K) row[k] = v[k] / sum;
       }
+      if (nl.on()) {
+        const uint64_t r = r0 + threadIdx.x;
+        const uint32_t label = nl.label(r);
+        nl.emit(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
+      }
     }
     __syncthreads();
     for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
@@ -138,7 +166,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
 template <int VPL, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
                                                                   const float *__restrict__ x,
-                                                                  float *__restrict__ y) {
+                                                                  float *__restrict__ y, RowNll nl) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int NG = VPL / W;  // groups per lane
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -174,15 +202,20 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
       s += v[i];
     }
     s = wave_sum(s);
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
       if (k < K) {
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          v[i * W + j] = v[i * W + j] / s;
+          if (nl.on()) nl.emit(r, K, label, k + uint32_t(j), v[i * W + j]);
+        }
         if (VEC) {
-          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k),
-                           f32x4{v[i * W] / s, v[i * W + 1] / s, v[i * W + 2] / s, v[i * W + 3] / s});
+          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
         } else {
-          yr[k] = v[i] / s;
+          yr[k] = v[i];
         }
       }
     }
@@ -204,7 +237,7 @@ __device__ inline void online_merge(float &m, float &s, float m2, float s2) {
 template <int VPT, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K, uint32_t R,
                                                                       const float *__restrict__ x,
-                                                                      float *__restrict__ y) {
+                                                                      float *__restrict__ y, RowNll nl) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int NG = VPT / W;
   __shared__ float lds[kBlock / kWave];
@@ -238,15 +271,20 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
       s += v[i];
     }
     s = block_sum(s, lds);
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
       if (k < K) {
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          v[i * W + j] = v[i * W + j] / s;
+          if (nl.on()) nl.emit(r, K, label, k + uint32_t(j), v[i * W + j]);
+        }
         if (VEC) {
-          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k),
-                           f32x4{v[i * W] / s, v[i * W + 1] / s, v[i * W + 2] / s, v[i * W + 3] / s});
+          store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
         } else {
-          yr[k] = v[i] / s;
+          yr[k] = v[i];
         }
       }
     }
@@ -256,7 +294,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
 // any K: one workgroup per row, the row streamed twice
 __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, uint32_t R,
                                                                    const float *__restrict__ x,
-                                                                   float *__restrict__ y) {
+                                                                   float *__restrict__ y, RowNll nl) {
   __shared__ float lds_m[kBlock / kWave], lds_s[kBlock / kWave];
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
@@ -288,12 +326,17 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
 #pragma unroll
     for (int w = 1; w < kBlock / kWave; ++w) online_merge(m, s, lds_m[w], lds_s[w]);
     __syncthreads();
-    for (uint32_t k = threadIdx.x; k < K; k += kBlock) yr[k] = expf(xr[k] - m) / s;
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
+      const float pr = expf(xr[k] - m) / s;
+      yr[k] = pr;
+      if (nl.on()) nl.emit(r, K, label, k, pr);
+    }
   }
 }
 
 void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float *x, float *y,
-                         CUstream_st *stream) {
+                         CUstream_st *stream, RowNll nl = RowNll{nullptr, nullptr, false}) {
   (void)checked_len(K, R, 1, symbol);
   if (K == 0 || R == 0) return;
   hipStream_t s = as_stream(stream);
@@ -311,13 +354,13 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     with_stream_policy(nt & kNtStore, [&](auto policy) {
       constexpr int NT = decltype(policy)::value;
       if (K <= 4) {
-        softmax_row_lds_kernel<4, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+        softmax_row_lds_kernel<4, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
       } else if (K <= 8) {
-        softmax_row_lds_kernel<8, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+        softmax_row_lds_kernel<8, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
       } else if (K <= 16) {
-        softmax_row_lds_kernel<16, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+        softmax_row_lds_kernel<16, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
       } else {
-        softmax_row_lds_kernel<32, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y);
+        softmax_row_lds_kernel<32, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
       }
     });
   } else if (K <= 64) {
@@ -326,7 +369,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     const uint32_t rows_per_block = kWavesPerBlock * (64u >> log2g);
     uint32_t blocks = (R + rows_per_block - 1) / rows_per_block;
     if (blocks > max_blocks) blocks = max_blocks;
-    softmax_row_subwave_kernel<<<blocks, kBlock, 0, s>>>(K, R, log2g, x, y);
+    softmax_row_subwave_kernel<<<blocks, kBlock, 0, s>>>(K, R, log2g, x, y, nl);
   } else if (K <= 2048) {
     uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > max_blocks) blocks = max_blocks;
@@ -335,10 +378,10 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   do {                                                                                   \
     if (vec) {                                                                           \
       with_stream_policy(nt, [&](auto policy) {                                          \
-        softmax_row_wave_kernel<VPL, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+        softmax_row_wave_kernel<VPL, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y, nl); \
       });                                                                                \
     } else {                                                                             \
-      softmax_row_wave_kernel<VPL, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);      \
+      softmax_row_wave_kernel<VPL, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y, nl);  \
     }                                                                                    \
   } while (0)
     if (K <= 256) {
@@ -358,10 +401,10 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   do {                                                                                   \
     if (vec) {                                                                           \
       with_stream_policy(nt, [&](auto policy) {                                          \
-        softmax_row_blockreg_kernel<VPT, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y); \
+        softmax_row_blockreg_kernel<VPT, true, decltype(policy)::value><<<blocks, kBlock, 0, s>>>(K, R, x, y, nl); \
       });                                                                                \
     } else {                                                                             \
-      softmax_row_blockreg_kernel<VPT, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y);  \
+      softmax_row_blockreg_kernel<VPT, false, 0><<<blocks, kBlock, 0, s>>>(K, R, x, y, nl); \
     }                                                                                    \
   } while (0)
     if (K <= 4096) {
@@ -371,7 +414,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     } else if (K <= 16384) {
       ANODE_ROW_BLOCKREG(64);
     } else {
-      softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y);
+      softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y, nl);
     }
 #undef ANODE_ROW_BLOCKREG
   }
@@ -868,6 +911,15 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_
   launch_softmax_nd_cat_nll_bwd<true>(__func__, prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, stream);
 }
 
+// Additive (no counterpart in the reference): row softmax and softmax_cat_nll in one pass over x (the recipe of
+// src/ops.rs:1172-1176 as one launch).  Writes the same probabilities and the same nll values as the two entry
+// points: the thread that stores the label's probability also writes -log of it.
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_fused_packed_f32(uint32_t dim0, uint32_t dim1, const float *x,
+                                                             const uint32_t *cat_data, float *softmax, float *nll,
+                                                             const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false});
+}
+
 // Additive (no counterpart in the reference): softmax_nd and softmax_nd_cat_nll in one pass over x.
 // Writes the same probabilities and the same nll values as the two separate entry points.
 ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
@@ -876,7 +928,9 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
                                                                 CUstream_st *stream) {
   const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
   if (len == 0) return;
-  if (prefix_dim > 1 && dim0 <= 32) {
+  if (prefix_dim == 1) {  // the class axis is contiguous: the row form
+    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false});
+  } else if (dim0 <= 32) {
     hipStream_t s = as_stream(stream);
     const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) && aligned16(nll);
     if (vec) {

@@ -9,7 +9,7 @@ from gpu_util import F32, assert_bit_exact, assert_close, call, dev, empty, host
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = [1, 3, 4, 5, 1023, 1024, 4099, (1 << 20) + 2]
+LENGTHS = [1, 3, 4, 5, 15, 16, 17, 1023, 1024, 4095, 4096, 4099, 4111, 8191, (1 << 20) + 2]
 
 
 @pytest.mark.parametrize("lo,hi", [(0.0, 1.0), (-1.0, 1.0), (-3.5, 2.25), (0.0, 255.0)])
@@ -187,6 +187,48 @@ def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
         assert_bit_exact(host(p2), host(p1), "fused softmax")
         assert_bit_exact(host(nll2), host(nll1), "fused nll")
         assert_close(host(p2), oracle.softmax_nd(P, C, N, x, f64=True), "fused softmax vs fp64", abs_floor=1e-30)
+
+
+ROW_FUSED_SHAPES = [(1, 5), (2, 7), (10, 32), (19, 513), (32, 600), (33, 9), (64, 300), (65, 3), (100, 17), (256, 5),
+                    (1000, 256), (1024, 3), (1025, 2), (2048, 2), (2049, 3), (4097, 2), (16385, 1), (40000, 1)]
+
+
+@pytest.mark.parametrize("K,R", ROW_FUSED_SHAPES)
+def test_fused_softmax_nll_rows_equals_the_two_launches(oracle, K, R):
+    # every row kernel (thread per row, lane group, wave, workgroup in registers, workgroup streamed)
+    g = np.random.default_rng(K * 3 + R)
+    x = (2 * g.standard_normal(K * R)).astype(F32)
+    lab = g.integers(0, K, R).astype(np.uint32)
+    if R > 4:
+        lab[1], lab[3] = K, 0xFFFFFFFF     # out of range: NaN
+        lab[2], lab[4] = 0, K - 1          # first and last class
+    for offset in (0, 1):
+        p1, nll1 = empty(K * R, offset=offset), empty(R, offset=offset)
+        call("anode_gpu_softmax_packed_deterministic_f32", K, R, dev(x, offset), p1)
+        call("anode_gpu_softmax_cat_nll_packed_f32", K, R, p1, dev(lab, offset), nll1)
+        p2, nll2 = empty(K * R, offset=offset), empty(R, offset=offset)
+        call("anode_gpu_softmax_cat_nll_fused_packed_f32", K, R, dev(x, offset), dev(lab, offset), p2, nll2)
+        assert_bit_exact(host(p2), host(p1), f"fused row softmax K={K}")
+        assert_bit_exact(host(nll2), host(nll1), f"fused row nll K={K}")
+        assert np.array_equal(np.isnan(host(nll2)), lab >= K)
+        assert_close(host(nll2), oracle.softmax_cat_nll(K, R, host(p2), lab, f64=True), "fused nll vs fp64", abs_floor=1e-6)
+        # the channel-axis entry point with one pixel per sample is the same thing
+        p3, nll3 = empty(K * R, offset=offset), empty(R, offset=offset)
+        call("anode_gpu_softmax_nd_cat_nll_fused_packed_f32", 1, K, R, dev(x, offset), dev(lab, offset), p3, nll3)
+        assert_bit_exact(host(p3), host(p1), "n-d fused with prefix 1")
+        assert_bit_exact(host(nll3), host(nll1), "n-d fused nll with prefix 1")
+
+
+def test_ref_fused_softmax_nll_known_answers():
+    # the reference's known answers (tests/test_gpu.rs:615-690) through the fused entry point
+    import math
+    p, nll = empty(64), empty(2)
+    call("anode_gpu_softmax_cat_nll_fused_packed_f32", 32, 2, dev(np.zeros(64, F32)), dev(np.array([12, 17], np.uint32)), p, nll)
+    assert np.all(host(p) == F32(1.0) / F32(32.0))
+    assert_close(host(nll), [math.log(32.0)] * 2, "nll", rel=1e-6)
+    call("anode_gpu_softmax_cat_nll_fused_packed_f32", 32, 2, dev(np.zeros(64, F32)), dev(np.array([12, 42], np.uint32)), p, nll)
+    h = host(nll)
+    assert np.isfinite(h[0]) and np.isnan(h[1]) and np.isnan(h.sum())
 
 
 def test_ref_online_average_quarter_steps(oracle):

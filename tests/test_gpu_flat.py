@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 SPECIALS = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.5, -2.25, 1e38, -1e38,
                      1.1754944e-38, -1.1754944e-38, 88.0, -88.0, 104.0, -104.0, 0.5, -0.5], F32)
 
-LENGTHS = [1, 2, 3, 4, 5, 63, 64, 255, 1024, 1027, 4096 * 3 + 1, 1 << 20, (1 << 20) + 3]
+LENGTHS = [1, 2, 3, 4, 5, 15, 16, 17, 63, 64, 255, 1024, 1027, 4095, 4096, 4111, 4096 * 3 + 1, 1 << 20, (1 << 20) + 3]
 
 # entry point -> (oracle map name, bit-exact against the fp32 restatement?)
 MAPS = {
