@@ -33,7 +33,7 @@ _SCALARS = {
     "void": None,
 }
 
-_DECL = re.compile(r"^\s*(void|int|uint32_t|size_t)\s+(anode_(?:gpu|host)_\w+)\s*\(([^;]*)\)\s*;", re.M)
+_DECL = re.compile(r"^\s*(void|int|uint32_t|size_t)\s+((?:anode_(?:gpu|host)|gpudevicemem)_\w+)\s*\(([^;]*)\)\s*;", re.M)
 
 
 def _ctype_of(param: str):

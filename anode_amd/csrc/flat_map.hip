@@ -40,6 +40,14 @@ struct Rcosh2Map {
     return 4.0f * t / (d * d);
   }
 };
+// Whitelisted for binding by the reference (build.rs:101-102) but left without a wrapper there; functor bodies at
+// flat_map.cu:242-278.  x <= 0 and NaN take the else branch.
+struct LogPositiveClipMap {
+  __device__ float operator()(float x, float) const { return (x > 0.0f) ? logf(x) : -__builtin_huge_valf(); }
+};
+struct PositiveReciprocalMap {
+  __device__ float operator()(float x, float) const { return (x > 0.0f) ? 1.0f / x : 0.0f; }
+};
 struct LeakyReluMap {
   float c;
   __device__ float operator()(float x, float) const {
@@ -291,6 +299,9 @@ ANODE_FLAT_MAP1(anode_gpu_unit_step_flat_map_f32, UnitStepMap)
 ANODE_FLAT_MAP1(anode_gpu_normal_cdf_flat_map_f32, NormalCdfMap)
 ANODE_FLAT_MAP1(anode_gpu_tanh_flat_map_f32, TanhMap)
 ANODE_FLAT_MAP1(anode_gpu_rcosh2_flat_map_f32, Rcosh2Map)
+// additive: named in the reference's bindgen whitelist (build.rs:101-102), never defined there
+ANODE_FLAT_MAP1(anode_gpu_log_positive_clip_flat_map_f32, LogPositiveClipMap)
+ANODE_FLAT_MAP1(anode_gpu_positive_reciprocal_flat_map_f32, PositiveReciprocalMap)
 
 ANODE_FLAT_MAP2(anode_gpu_positive_clip_flat_map_bwd_f32, PositiveClipBwdMap)
 ANODE_FLAT_MAP2(anode_gpu_logistic_flat_map_bwd_f32, LogisticBwdMap)

@@ -21,7 +21,7 @@
 // (hipHostMalloc), never registered.
 #pragma once
 
-#include "anode_amd/host/ops_gpu.hpp"
+#include "anode_amd/host/arrays.hpp"
 
 #include <hip/hip_runtime.h>
 

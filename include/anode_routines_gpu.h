@@ -199,6 +199,14 @@ void anode_gpu_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, u
 /* lib.h:423-430 (commented out).  y[b] = sum_{a,c} x[a,b,c]^2 */
 void anode_gpu_square_sum_Iabc_Ob_packed_deterministic_f32(uint32_t reduce_inner_dim, uint32_t mid_dim, uint32_t reduce_outer_dim, const float *x, float *y, ANODE_LAUNCH_TAIL);
 
+/* ---- whitelisted for binding by the reference (build.rs:101-102) but never defined there; functor bodies at
+ *      flat_map.cu:242-278 ---- */
+
+/* y = x > 0 ? log(x) : -inf   (NaN -> -inf: the comparison is false) */
+void anode_gpu_log_positive_clip_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* y = x > 0 ? 1 / x : 0 */
+void anode_gpu_positive_reciprocal_flat_map_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+
 /* ---- no counterpart in the reference ---- */
 
 /* Inverse of dequantize: scale = (hi-lo)/255; y = clamp(rint((x-lo)/scale), 0, 255), round half to even, NaN -> 0. */
@@ -252,7 +260,8 @@ void anode_gpu_softmax_nd_cat_nll_bwd_ignore_packed_accumulate_f32(uint32_t pref
 
 /* ---- the neighbours anode takes from its sibling library gpudevicemem (source not part of the reference tree) ----
  * Signatures follow the call sites in src/ops_gpu.rs; the arithmetic is the closed form those call sites imply.
- * Exported under this library's prefix so that both libraries can be linked together. */
+ * Exported under this library's prefix; the five that anode calls directly over FFI are repeated below under
+ * their gpudevicemem names. */
 
 /* src/ops_gpu.rs:7486-7492 (gpudevicemem_sum_packed_deterministic_f32): y[0] = sum_i x[i]; fp64 accumulation in a fixed order. */
 void anode_gpu_sum_packed_deterministic_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
@@ -274,6 +283,21 @@ void anode_gpu_mult_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAU
 void anode_gpu_is_nonzero_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
 /* src/ops_gpu.rs:5886 (online_add): y[i] = fma(rate, x[i], y[i]). */
 void anode_gpu_online_add_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
+
+/* The same five under the link names anode calls them by, directly over FFI, for a build that has no ROCm
+ * gpudevicemem yet.  In the static archive they sit in an object of their own (gpudevicemem_names.o), which the
+ * linker only pulls in while one of these names is still undefined: list a real gpudevicemem before this library
+ * and its definitions win; never force-load (--whole-archive) both. */
+/* src/ops_gpu.rs:7486-7492 */
+void gpudevicemem_sum_packed_deterministic_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7499-7505 */
+void gpudevicemem_sum_packed_accumulate_deterministic_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7595-7601, :7706-7712 */
+void gpudevicemem_bcast_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:7608-7614, :7719-7725 */
+void gpudevicemem_bcast_packed_accumulate_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:9592-9600 */
+void gpudevicemem_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32(uint32_t inner_dim, uint32_t outer_dim, const float *x, const float *rdivisor, float *y, ANODE_LAUNCH_TAIL);
 
 /* The host-side rule itself (src/utils/mod.rs:31-41), for logits already on the host: first index of the strict
  * maximum starting from (-inf, 0); NaN never selected.  xs is a HOST pointer. */

@@ -86,13 +86,16 @@ def rms(a):
 
 
 def assert_close(got, ref64, what="", rel=REL, abs_floor=0.0):
-    """|got - ref| <= rel*|ref| + abs_floor, NaNs must coincide."""
+    """|got - ref| <= rel*|ref| + abs_floor; NaNs must coincide, infinities must be equal."""
     got = np.asarray(got, np.float64)
     ref64 = np.asarray(ref64, np.float64)
     assert got.shape == ref64.shape, (what, got.shape, ref64.shape)
     nan_g, nan_r = np.isnan(got), np.isnan(ref64)
     assert np.array_equal(nan_g, nan_r), f"{what}: NaN pattern differs ({nan_g.sum()} vs {nan_r.sum()})"
     ok = ~nan_r
+    inf_r = np.isinf(ref64)
+    assert np.array_equal(got[inf_r], ref64[inf_r]), f"{what}: infinities differ"
+    ok &= ~inf_r
     err = np.abs(got[ok] - ref64[ok])
     bound = rel * np.abs(ref64[ok]) + abs_floor
     if not np.all(err <= bound):

@@ -1,9 +1,9 @@
 // Native caller harness: drives the library the way anode's Rust host side
-// does -- through the C++ mirror of src/ops_gpu.rs (anode_amd/host/ops_gpu.hpp),
+// does -- through the C++ mirror of src/ops_gpu.rs (tests/native/ops_gpu.hpp),
 // linked against the STATIC archive libanode_routines_gpu.a -- and re-runs the
 // reference's own GPU tests for this path (tests/test_gpu.rs:595-758) plus the
 // batch-norm recipe, checked against the CPU oracle.  Test infrastructure.
-#include "anode_amd/host/ops_gpu.hpp"
+#include "tests/native/ops_gpu.hpp"
 
 #include <cmath>
 #include <cstdio>

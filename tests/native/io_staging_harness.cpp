@@ -4,6 +4,7 @@
 // job (synchronous pageable copies + a separate operator, src/io_gpu.rs:286-330)
 // and prints the host-buffer-inclusive rates as one JSON line.  Test infrastructure.
 #include "anode_amd/host/io_gpu.hpp"
+#include "tests/native/ops_gpu.hpp"
 
 #include <chrono>
 #include <cmath>

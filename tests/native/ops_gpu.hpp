@@ -1,4 +1,4 @@
-// Host side above the C ABI, in C++: the caller layer of anode's
+// Test harness, not product.  Host side above the C ABI, in C++: the caller layer of anode's
 // src/ops_gpu.rs for the operators of routines_gpu, with the same operator
 // names, the same dimension mapping, the same Assign / Accumulate dispatch and
 // the same failure behaviour (the reference's `unimplemented!()` and `assert!`
@@ -11,117 +11,11 @@
 // first, plus a batch size), described here by a device pointer and a Shape.
 #pragma once
 
-#define ANODE_DEFINE_KERNEL_CONFIG
-#include "../../include/anode_routines_gpu.h"
-
-#include <hip/hip_runtime.h>
-
-#include <cstddef>
-#include <cstdint>
-#include <stdexcept>
-#include <string>
+#include "anode_amd/host/arrays.hpp"
 
 namespace anode_host {
 
-// src/lib.rs:1810-1813
-enum class WriteCap { Assign, Accumulate };
-
-// the reference's `unimplemented!()`
-struct Unimplemented : std::logic_error {
-  explicit Unimplemented(const std::string &what) : std::logic_error("unimplemented: " + what) {}
-};
-
-// src/ops_gpu.rs:57-61: sizes must fit the ABI's u32
-inline uint32_t sz2uint(size_t sz) {
-  if (sz > 0xffffffffull) throw std::overflow_error("sz2uint: size does not fit in u32");
-  return uint32_t(sz);
-}
-
-// What the Rust callers take from their connection: conn.cuda_stream() and
-// conn.cuda_kernel_config() (src/ops_gpu.rs:670-679).
-struct GPUDeviceConn {
-  hipStream_t stream = nullptr;
-  KernelConfig cfg{1024, 1024};
-  const KernelConfig *cuda_kernel_config() const { return &cfg; }
-  CUstream_st *cuda_stream() const { return reinterpret_cast<CUstream_st *>(stream); }
-};
-
-// Non-batch dimensions (fastest first) and the outer batch size.
-struct Shape {
-  size_t size[4] = {1, 1, 1, 1};
-  int nd = 1;
-  size_t batch = 1;
-  size_t index_at(int i) const { return i < nd ? size[i] : batch; }  // the batch is the last axis
-  size_t flat_len_upto(int n) const {                                // product of the first n axes
-    size_t p = 1;
-    for (int i = 0; i < n; ++i) p *= size[i];
-    return p;
-  }
-  size_t flat_len() const { return flat_len_upto(nd) * batch; }
-};
-
-template <typename T>
-struct DeviceArray {
-  T *dptr = nullptr;
-  Shape shape;
-  bool packed = true;  // only packed arrays are implemented, as in the reference
-  bool is_packed() const { return packed; }
-  const T *as_dptr() const { return dptr; }
-  T *as_mut_dptr() const { return dptr; }
-};
-
-inline DeviceArray<float> array1d(float *p, size_t n) {
-  DeviceArray<float> a;
-  a.dptr = p;
-  a.shape.size[0] = n;
-  a.shape.nd = 1;
-  return a;
-}
-
-// [d0, batch]: GPUDeviceOuterBatchArray1d
-template <typename T>
-inline DeviceArray<T> obatch1d(T *p, size_t d0, size_t batch) {
-  DeviceArray<T> a;
-  a.dptr = p;
-  a.shape.size[0] = d0;
-  a.shape.nd = 1;
-  a.shape.batch = batch;
-  return a;
-}
-
-// [W, H, C, batch]: GPUDeviceOuterBatchArray3d (NCHW memory)
-template <typename T>
-inline DeviceArray<T> obatch3d(T *p, size_t w, size_t h, size_t c, size_t batch) {
-  DeviceArray<T> a;
-  a.dptr = p;
-  a.shape.size[0] = w;
-  a.shape.size[1] = h;
-  a.shape.size[2] = c;
-  a.shape.nd = 3;
-  a.shape.batch = batch;
-  return a;
-}
-
-// [X, Y, Z, C, batch]: GPUDeviceOuterBatchArray4d (NCDHW memory)
-template <typename T>
-inline DeviceArray<T> obatch4d(T *p, size_t x, size_t y, size_t z, size_t c, size_t batch) {
-  DeviceArray<T> a;
-  a.dptr = p;
-  a.shape.size[0] = x;
-  a.shape.size[1] = y;
-  a.shape.size[2] = z;
-  a.shape.size[3] = c;
-  a.shape.nd = 4;
-  a.shape.batch = batch;
-  return a;
-}
-
 namespace detail {
-template <typename... A>
-inline void require_packed(const char *op, const A &...arrays) {
-  const bool packed = (arrays.is_packed() && ...);
-  if (!packed) throw Unimplemented(std::string(op) + ": non-packed arrays");
-}
 // (dim0, dim1, dim2) = (flat_len of the spatial axes, channels, batch): src/ops_gpu.rs:3764-3766, 4911-4913
 struct Dims3 {
   uint32_t d0, d1, d2;
@@ -465,9 +359,9 @@ struct BatchSumOp {  // src/ops_gpu.rs:7478-7505: x is a batch of scalars, y one
     detail::require_packed("BatchSumOp", x, y);
     const uint32_t len = sz2uint(x.shape.flat_len());
     if (cap == WriteCap::Assign) {
-      anode_gpu_sum_packed_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+      gpudevicemem_sum_packed_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
     } else {
-      anode_gpu_sum_packed_accumulate_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
+      gpudevicemem_sum_packed_accumulate_deterministic_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(),
                                                         conn.cuda_stream());
     }
   }
@@ -478,9 +372,9 @@ struct BatchBroadcastOp {  // src/ops_gpu.rs:7585-7614 (and :7706-7719): x is on
     detail::require_packed("BatchBroadcastOp", x, y);
     const uint32_t len = sz2uint(y.shape.flat_len());
     if (cap == WriteCap::Assign) {
-      anode_gpu_bcast_packed_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+      gpudevicemem_bcast_packed_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
     } else {
-      anode_gpu_bcast_packed_accumulate_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
+      gpudevicemem_bcast_packed_accumulate_f32(len, x.as_dptr(), y.as_mut_dptr(), conn.cuda_kernel_config(), conn.cuda_stream());
     }
   }
 };
@@ -492,7 +386,7 @@ struct FlatBroadcastRdivOp {  // src/ops_gpu.rs:9575-9605: y[.., b] = x[.., b] /
     if (cap != WriteCap::Assign) throw Unimplemented("FlatBroadcastRdivOp: Accumulate");  // :9602
     if (x.shape.batch != rdivisor.shape.batch) throw std::invalid_argument("FlatBroadcastRdivOp: batch sizes differ");  // :9578
     const size_t batch = x.shape.batch;
-    anode_gpu_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32(sz2uint(batch ? x.shape.flat_len() / batch : 0), sz2uint(batch),
+    gpudevicemem_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32(sz2uint(batch ? x.shape.flat_len() / batch : 0), sz2uint(batch),
                                                       x.as_dptr(), rdivisor.as_dptr(), y.as_mut_dptr(),
                                                       conn.cuda_kernel_config(), conn.cuda_stream());
   }

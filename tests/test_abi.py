@@ -106,6 +106,37 @@ def test_static_archive_defines_every_reference_symbol():
         assert name in defined
 
 
+GPUDEVICEMEM_NAMES = {  # the argument lists of the direct FFI calls at src/ops_gpu.rs:7486-7505, 7595-7614, 9592-9600
+    "gpudevicemem_sum_packed_deterministic_f32": "upp",
+    "gpudevicemem_sum_packed_accumulate_deterministic_f32": "upp",
+    "gpudevicemem_bcast_packed_f32": "upp",
+    "gpudevicemem_bcast_packed_accumulate_f32": "upp",
+    "gpudevicemem_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32": "uuppp",
+}
+
+
+def test_gpudevicemem_link_names_are_exported_from_an_object_of_their_own():
+    protos = _lib.parse_header()
+    for name, kinds in GPUDEVICEMEM_NAMES.items():
+        restype, argtypes, names = protos[name]
+        assert restype is None and "".join(_KIND[t] for t in argtypes) == kinds + "pp" and names[-2:] == ["cfg", "stream"]
+    assert set(GPUDEVICEMEM_NAMES) <= _nm_defined(_lib.LIBRARY_PATH, dynamic=True)
+    # in the archive they are the only definitions of their member, so a link that already has a gpudevicemem
+    # never pulls them in
+    out = subprocess.run(["nm", "-g", "--defined-only", _lib.STATIC_LIBRARY_PATH], check=True, capture_output=True,
+                         text=True).stdout
+    member, by_member = None, {}
+    for line in out.splitlines():
+        if line.endswith(".o:"):
+            member = line[:-1]
+        elif " T " in line:
+            by_member.setdefault(member, set()).add(line.split()[-1])
+    owners = [m for m, syms in by_member.items() if syms & set(GPUDEVICEMEM_NAMES)]
+    assert owners == ["gpudevicemem_names.o"], owners
+    extern_c = {s for s in by_member["gpudevicemem_names.o"] if not s.startswith("_Z") and not s.startswith("__hip")}
+    assert extern_c == set(GPUDEVICEMEM_NAMES), extern_c
+
+
 def test_library_loads_and_reports_symbol_count():
     lib = _lib.load()
     assert lib.symbol("anode_gpu_reference_symbol_count")() == 46

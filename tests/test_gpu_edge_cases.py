@@ -16,7 +16,7 @@ from gpu_util import F32, assert_bit_exact, assert_close, call, dev, host
 pytestmark = pytest.mark.gpu
 
 SENTINEL = 12345.0
-WRITES_ON_EMPTY = {"anode_gpu_sum_packed_deterministic_f32"}
+WRITES_ON_EMPTY = {"anode_gpu_sum_packed_deterministic_f32", "gpudevicemem_sum_packed_deterministic_f32"}
 
 
 def _entry_points():

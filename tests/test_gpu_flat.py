@@ -26,6 +26,9 @@ MAPS = {
     "anode_gpu_normal_cdf_flat_map_f32": ("normal_cdf", False),
     "anode_gpu_tanh_flat_map_f32": ("tanh", False),
     "anode_gpu_rcosh2_flat_map_f32": ("rcosh2", False),
+    # whitelisted by the reference's build.rs:101-102, defined only here (functors: flat_map.cu:242-278)
+    "anode_gpu_log_positive_clip_flat_map_f32": ("log_positive_clip", False),
+    "anode_gpu_positive_reciprocal_flat_map_f32": ("positive_reciprocal", True),  # one correctly rounded division
 }
 
 

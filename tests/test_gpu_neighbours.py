@@ -101,6 +101,41 @@ def test_flat_bcast_rdiv(inner, outer):
         assert_bit_exact(host(y), oracle.flat_bcast_rdiv(inner, outer, x, r), "rdiv")
 
 
+def test_gpudevicemem_link_names(oracle=oracle):
+    # the five entry points anode calls by their gpudevicemem names (src/ops_gpu.rs:7486-7505, 7595-7614, 9592-9600):
+    # against the oracle / numpy, and bit for bit against the anode_gpu_* twins they forward to
+    g = np.random.default_rng(11)
+    n = 4099
+    x = (1 + g.standard_normal(n)).astype(F32)
+    y = dev(np.array([7.0], F32))
+    call("gpudevicemem_sum_packed_deterministic_f32", n, dev(x), y)
+    assert_close(host(y), [oracle.sum_packed(x)], "sum", abs_floor=1e-6 * np.sqrt(n))
+    twin = dev(np.array([7.0], F32))
+    call("anode_gpu_sum_packed_deterministic_f32", n, dev(x), twin)
+    assert_bit_exact(host(y), host(twin), "sum twin")
+    first = host(y).copy()
+    y = dev(np.array([7.0], F32))
+    call("gpudevicemem_sum_packed_accumulate_deterministic_f32", n, dev(x), y)
+    assert_bit_exact(host(y), F32(7.0) + first, "sum accumulate")
+    call("gpudevicemem_sum_packed_deterministic_f32", 10, dev(np.ones(10, F32)), y)
+    assert host(y)[0] == F32(10.0)    # the value the reference's sum-join test expects (tests/test_gpu.rs:302-353)
+
+    s, y0 = np.array([1.625], F32), g.standard_normal(n).astype(F32)
+    y = empty(n)
+    call("gpudevicemem_bcast_packed_f32", n, dev(s), y)
+    assert_bit_exact(host(y), np.full(n, s[0], F32), "bcast")
+    y = dev(y0)
+    call("gpudevicemem_bcast_packed_accumulate_f32", n, dev(s), y)
+    assert_bit_exact(host(y), y0 + s[0], "bcast accumulate")
+
+    inner, outer = 1000, 3
+    xr = g.standard_normal(inner * outer).astype(F32)
+    r = (0.5 + g.random(outer)).astype(F32)
+    y = empty(inner * outer)
+    call("gpudevicemem_flat_bcast_rdiv_I1ab_I2b_Oab_packed_f32", inner, outer, dev(xr), dev(r), y)
+    assert_bit_exact(host(y), oracle.flat_bcast_rdiv(inner, outer, xr, r), "rdiv")
+
+
 @pytest.mark.parametrize("K,R", [(10, 32), (1000, 5), (1, 3), (33, 64)])
 def test_row_nll_ignore(K, R):
     g = np.random.default_rng(K * R)
