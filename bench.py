@@ -54,26 +54,58 @@ class Launch:
 
 # HBM bytes per launch from hardware counters, keyed by (symbol, workload group): two rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain copy
-# of known size in the same run (--copy-calibration): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  A launch that is not
-# listed reports null.
+# of known size in the same run (--copy-calibration): FETCH_SIZE x 2.000, WRITE_SIZE x 1.000.  These are the figures
+# of the profile named in TRAFFIC_SOURCE, not re-measured by this run; a launch that is not listed reports null.
+TRAFFIC_SOURCE = "profiles/bench_step_dominant_kernels_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not re-measured in this run)"
 MEASURED_TRAFFIC = {
-    # 802 838 KiB fetched, 802 816 KiB written; algorithmic bytes are 2 466 250 752
-    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2a"): 2466122509,
+    # (symbol, group): bytes
 }
+
+
+class Draws:
+    """Synthetic inputs drawn as the measurement spec prescribes: numpy.random.default_rng(0) (PCG64), normals and
+    uniforms drawn in float64 and cast to float32, labels from integers(); one generator for the whole workload,
+    consumed in the order configs 1, 2a, 2b, 3a, 3b, 4 (within a config: the order the arrays are listed in
+    `config.inputs`).  Arrays are produced in chunks so that an 822 MB tensor never needs its float64 image on the
+    host at once."""
+
+    CHUNK = 1 << 24
+
+    def __init__(self, torch, np):
+        self.torch, self.np = torch, np
+        self.rng = np.random.default_rng(0)
+
+    def _fill(self, out, make):
+        n = out.numel()
+        for lo in range(0, n, self.CHUNK):
+            m = min(self.CHUNK, n - lo)
+            out[lo:lo + m].copy_(self.torch.from_numpy(make(m)))
+        return out
+
+    def normal(self, out, mean=0.0, std=1.0):
+        np = self.np
+        return self._fill(out, lambda m: (mean + std * self.rng.standard_normal(m)).astype(np.float32))
+
+    def uniform(self, out, lo, hi):
+        np = self.np
+        return self._fill(out, lambda m: (lo + (hi - lo) * self.rng.random(m)).astype(np.float32))
+
+    def integers(self, out, hi):
+        np = self.np
+        if out.dtype == self.torch.uint8:
+            return self._fill(out, lambda m: self.rng.integers(0, hi, m, dtype=np.uint8))
+        return self._fill(out, lambda m: self.rng.integers(0, hi, m).astype(np.uint32).view(np.int32))
+
+    def mask(self, n, prob):
+        out = self.torch.empty(n, device="cuda", dtype=self.torch.bool)
+        return self._fill(out, lambda m: self.rng.random(m) < prob)
 
 
 def build_workload(torch, only, copy_calibration=False):
     """All device buffers and the launch list of one step."""
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
+    import numpy as np
 
-    def randn(n, mean=0.0, std=1.0):
-        t = torch.randn(n, device="cuda", generator=g)
-        if std != 1.0:
-            t.mul_(std)
-        if mean != 0.0:
-            t.add_(mean)
-        return t
+    draw = Draws(torch, np)
 
     def empty(n, dtype=torch.float32):
         return torch.empty(n, device="cuda", dtype=dtype)
@@ -86,29 +118,73 @@ def build_workload(torch, only, copy_calibration=False):
 
     if copy_calibration:
         n = 64 * 1024 * 1024  # 256 MiB in, 256 MiB out
-        src, dst = randn(n), empty(n)
+        src, dst = torch.randn(n, device="cuda"), empty(n)
         launches.append(Launch("copy_calibration", "anode_gpu_copy_flat_map_f32", (n, src, dst), 8 * n, n))
+
+    # ---- device arrays are allocated in launch order (config 1, 2a, 2b, 4, 3a, 3b: x, dy, y, dx per layer) and then
+    # ---- filled by draws in config order (1, 2a, 2b, 3a, 3b, 4)
+    n1 = 256 * 3 * 224 * 224
+    cast = want("cast_cfg1")
+    q1 = empty(n1, torch.uint8) if cast else None
+    yf1, yu1 = (empty(n1), empty(n1, torch.int32)) if cast else (None, None)
+    z1, zq1 = (empty(n1), empty(n1, torch.uint8)) if cast else (None, None)
+    bn_shapes = {"cfg2a": (112 * 112, 64, 256, 2.0, 3.0), "cfg2b": (49, 2048, 256, 2.0, 3.0),
+                 "cfg4": (128 * 128 * 128, 32, 2, 0.0, 1.0)}
+    bn_data = {}
+    for tag, (S, C, N, _, _) in bn_shapes.items():
+        if want(f"bn_fwd_{tag}") or want(f"bn_bwd_{tag}") or (tag == "cfg4" and want("relu_cfg4")):
+            n = S * C * N
+            bn_data[tag] = {"x": empty(n), "dy": empty(n), "y": empty(n), "dx": empty(n),
+                            "gamma": torch.ones(C, device="cuda"), "beta": torch.zeros(C, device="cuda")}
+    sm3a = sm3b = None
+    if want("softmax_cfg3a"):
+        sm3a = (empty(1000 * 256), empty(256, torch.int32))
+    if want("softmax_cfg3b"):
+        sm3b = (empty(512 * 1024 * 19 * 8), empty(512 * 1024 * 8, torch.int32))
+
+    if cast:
+        draw.integers(q1, 256)
+        draw.normal(z1)
+    for tag in ("cfg2a", "cfg2b"):
+        if tag in bn_data:
+            _, _, _, mean, std = bn_shapes[tag]
+            draw.normal(bn_data[tag]["x"], mean, std)
+            draw.normal(bn_data[tag]["dy"])
+            draw.uniform(bn_data[tag]["gamma"], 0.5, 1.5)
+            draw.normal(bn_data[tag]["beta"], 0.0, 0.1)
+    if sm3a is not None:
+        draw.normal(sm3a[0], 0.0, 2.0)          # "N(0,4)": variance 4, sigma 2
+        draw.integers(sm3a[1], 1000)
+    if sm3b is not None:
+        draw.normal(sm3b[0])
+        draw.integers(sm3b[1], 19)
+        sm3b[1][draw.mask(512 * 1024 * 8, 0.05)] = 255   # 5 % ignore-index
+    if "cfg4" in bn_data:                        # gamma = 1, beta = 0
+        draw.normal(bn_data["cfg4"]["x"])
+        draw.normal(bn_data["cfg4"]["dy"])
 
     # ---- config 1: u8 image batch [256,3,224,224] -> f32 / u32 -------------------
     if want("cast_cfg1"):
-        n = 256 * 3 * 224 * 224
-        q = torch.randint(0, 256, (n,), device="cuda", dtype=torch.uint8, generator=g)
-        yf, yu = empty(n), empty(n, torch.int32)
-        launches.append(Launch("cast_cfg1", "anode_gpu_dequantize_u8_packed_f32", (n, 0.0, 1.0, q, yf), 5 * n, n))
-        launches.append(Launch("cast_cfg1", "anode_gpu_upcast_u8_packed_u32", (n, q, yu), 5 * n, n))
-        # per-channel image normalisation in one pass, and f32 -> u8 quantisation of an N(0,1) tensor
+        n, yf, yu, zq = n1, yf1, yu1, zq1
+        launches.append(Launch("cast_cfg1", "anode_gpu_dequantize_u8_packed_f32", (n, 0.0, 1.0, q1, yf), 5 * n, n))
+        launches.append(Launch("cast_cfg1", "anode_gpu_upcast_u8_packed_u32", (n, q1, yu), 5 * n, n))
+        # what the config names beyond the reference's two casts: per-channel image normalisation in one pass, and
+        # f32 -> u8 quantisation of an N(0,1) tensor (scale 8/255, zero point at -4; parity unpinned by the
+        # reference, which has no such kernel)
         a = torch.tensor([1 / (255 * 0.229), 1 / (255 * 0.224), 1 / (255 * 0.225)], device="cuda")
         b = torch.tensor([-0.485 / 0.229, -0.456 / 0.224, -0.406 / 0.225], device="cuda")
-        z, zq = randn(n), empty(n, torch.uint8)
         fused.append(Launch("fused_cast_cfg1", "anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32",
-                            (224 * 224, 3, 256, a, b, q, yf), 5 * n, n))
-        fused.append(Launch("fused_cast_cfg1", "anode_gpu_quantize_u8_packed_f32", (n, -4.0, 4.0, z, zq), 5 * n, n))
+                            (224 * 224, 3, 256, a, b, q1, yf), 5 * n, n))
+        fused.append(Launch("fused_cast_cfg1", "anode_gpu_quantize_u8_packed_f32", (n, -4.0, 4.0, z1, zq), 5 * n, n))
 
     # ---- configs 2a, 2b, 4: batch norm forward + backward -------------------------
-    def bn(tag, S, C, N, mean, std, relu=False):
+    def bn(tag, relu=False):
+        if tag not in bn_data:
+            return None
+        S, C, N, _, _ = bn_shapes[tag]
+        t = bn_data[tag]
+        x, dy, y, dx, gamma, beta = t["x"], t["dy"], t["y"], t["dx"], t["gamma"], t["beta"]
         n = S * C * N
-        x, dy = randn(n, mean, std), randn(n)
-        y, dx = empty(n), empty(n)
         m, v, dm, dv = empty(C), empty(C), empty(C), empty(C)
         d = (S, C, N)
         f, b = f"bn_fwd_{tag}", f"bn_bwd_{tag}"
@@ -136,35 +212,47 @@ def build_workload(torch, only, copy_calibration=False):
                                 (*d, dy, x, m2, v2, mask, dm2, dv2), (12 if relu else 8) * n, n))
             fused.append(Launch(f"fused_{b}", "anode_gpu_batch_norm_bwd_apply_3d1_packed_f32",
                                 (*d, dy, x, m2, v2, dm2, dv2, mask, dx2), (16 if relu else 12) * n, n))
+            if not relu:
+                # the layer the config words: batch statistics, normalise with gamma / beta, running statistics with
+                # momentum 0.1 (src/ops.rs:1002-1003: online_average of the mean and of var + eps)
+                rm, rv = torch.zeros(C, device="cuda"), torch.ones(C, device="cuda")
+                g_ = f"affine_{f}"
+                fused.append(Launch(g_, "anode_gpu_batch_mean_var_3d1_packed_f32", (*d, 1e-5, x, m2, v2), 4 * n, n))
+                fused.append(Launch(g_, "anode_gpu_batch_norm_affine_3d1_packed_f32", (*d, x, m2, v2, gamma, beta, y2), 8 * n, n))
+                fused.append(Launch(g_, "anode_gpu_online_average_packed_f32", (C, 0.1, m2, rm), 12 * C, C))
+                fused.append(Launch(g_, "anode_gpu_online_average_packed_f32", (C, 0.1, v2, rv), 12 * C, C))
         return x, dy, y, dx
 
-    bn("cfg2a", 112 * 112, 64, 256, 2.0, 3.0)
-    bn("cfg2b", 49, 2048, 256, 2.0, 3.0)
-    x4, dy4, y4, dx4 = bn("cfg4", 128 * 128 * 128, 32, 2, 0.0, 1.0, relu=True)
-    if want("relu_cfg4"):
+    bn("cfg2a")
+    bn("cfg2b")
+    r4 = bn("cfg4", relu=True)
+    if want("relu_cfg4") and r4 is not None:
+        x4, dy4, y4, dx4 = r4
         n = x4.numel()
         # ReLU after BN, in place (examples/bench_unet3d.rs:103), and its mask backward
         launches.append(Launch("relu_cfg4", "anode_gpu_positive_clip_flat_map_f32", (n, y4, y4), 8 * n, n))
         launches.append(Launch("relu_cfg4", "anode_gpu_positive_clip_flat_map_bwd_f32", (n, dy4, y4, dx4), 12 * n, n))
 
     # ---- config 3a: row softmax + NLL [256,1000] ---------------------------------
-    if want("softmax_cfg3a"):
+    if sm3a is not None:
         K, R = 1000, 256
-        x = randn(K * R, 0.0, 2.0)
-        lab = torch.randint(0, K, (R,), device="cuda", dtype=torch.int32, generator=g)
+        x, lab = sm3a
         p, nll, dx, dy = empty(K * R), empty(R), empty(K * R), torch.ones(R, device="cuda")
         launches.append(Launch("softmax_cfg3a", "anode_gpu_softmax_packed_block_f32", (K, R, x, p), 8 * K * R, K * R))
         launches.append(Launch("softmax_cfg3a", "anode_gpu_softmax_cat_nll_packed_f32", (K, R, p, lab, nll), 12 * R, R))
         launches.append(Launch("softmax_cfg3a", "anode_gpu_softmax_cat_nll_bwd_packed_f32", (K, R, dy, p, lab, dx),
                                8 * K * R + 8 * R, K * R))
+        p2, nll2, dx2 = empty(K * R), empty(R), empty(K * R)
+        fused.append(Launch("fused_softmax_cfg3a", "anode_gpu_softmax_cat_nll_fused_packed_f32",
+                            (K, R, x, lab, p2, nll2), 8 * K * R + 8 * R, K * R))
+        fused.append(Launch("fused_softmax_cfg3a", "anode_gpu_softmax_cat_nll_bwd_packed_f32", (K, R, dy, p2, lab, dx2),
+                            8 * K * R + 8 * R, K * R))
 
     # ---- config 3b: channel-axis softmax + NLL [8,19,512,1024] -------------------
-    if want("softmax_cfg3b"):
+    if sm3b is not None:
         P, C, N = 512 * 1024, 19, 8
         n = P * C * N
-        x = randn(n)
-        lab = torch.randint(0, C, (P * N,), device="cuda", dtype=torch.int32, generator=g)
-        lab[torch.rand(P * N, device="cuda", generator=g) < 0.05] = 255
+        x, lab = sm3b
         p, nll, dx, dy = empty(n), empty(P * N), empty(n), torch.ones(P * N, device="cuda")
         launches.append(Launch("softmax_cfg3b", "anode_gpu_softmax_nd_packed_f32", (P, C, N, x, p), 8 * n, n))
         launches.append(Launch("softmax_cfg3b", "anode_gpu_softmax_nd_cat_nll_packed_f32", (P, C, N, p, lab, nll),
@@ -388,7 +476,7 @@ def small_shape_latency(torch, gpu, groups, passes=100):
     return out
 
 
-def small_shape_groups(torch, launches):
+def small_shape_groups(torch, launches, fused=()):
     """Config 0 (BN on [32,16,28,28], softmax + NLL on [32,10]) and the config 3a launches of the step."""
     def empty(n):
         return torch.empty(n, device="cuda")
@@ -417,6 +505,9 @@ def small_shape_groups(torch, launches):
     cfg3a = [l for l in launches if l.group == "softmax_cfg3a"]
     if cfg3a:
         groups["softmax_nll_cfg3a"] = cfg3a
+    cfg3a_fused = [l for l in fused if l.group == "fused_softmax_cfg3a"]
+    if cfg3a_fused:
+        groups["softmax_nll_cfg3a_fused_fwd"] = cfg3a_fused  # softmax + NLL in one launch, then the backward
     return groups
 
 
@@ -426,7 +517,9 @@ def cpu_baseline():
 
     from oracle import binding as o
 
-    threads = min(16, os.cpu_count() or 1)
+    host_cpus = os.cpu_count() or 1
+    omp_default = o.max_threads()
+    threads = min(16, host_cpus)  # the GPU box grants 16 cores per GPU whatever nproc shows
     o.set_threads(threads)
     g = np.random.default_rng(0)
     F32 = np.float32
@@ -495,6 +588,8 @@ def cpu_baseline():
         "value": round(total_bytes / total_s / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "host_cpus_reported": host_cpus,
+        "omp_max_threads_default": omp_default,
         "single_thread": {"value": round(single_gbps, 3), "unit": "GB/s", "cores": 1, "seconds": round(single_s, 2)},
         "kind": "port",
         "sample": "fp32 CPU restatement, OpenMP: BN fwd+bwd (9 launches) on [64,64,112,112]; softmax_nd+NLL+bwd on "
@@ -588,7 +683,15 @@ def main():
         "alg_bytes_per_launch": dom.alg_bytes,
         "avg_launch_us": round(dom_s * 1e6, 2),
         "traffic": MEASURED_TRAFFIC.get((dom.symbol, dom.group)),
+        "traffic_source": TRAFFIC_SOURCE,
     }
+    # the same counters for the dominant kernel of every config (bytes per launch; ratio to the algorithmic bytes)
+    traffic_by_kernel = []
+    for l in launches:
+        t = MEASURED_TRAFFIC.get((l.symbol, l.group))
+        if t is not None:
+            traffic_by_kernel.append({"group": l.group, "symbol": l.symbol.replace("anode_gpu_", ""),
+                                      "alg_bytes": l.alg_bytes, "traffic": t, "ratio": round(t / l.alg_bytes, 3)})
 
     groups = {}
     for l, t in zip(launches, med):
@@ -608,7 +711,7 @@ def main():
             gpu.call(l.symbol, *l.args)
         torch.cuda.synchronize()
         ftimes = [[] for _ in fused]
-        for _ in range(5):
+        for _ in range(10):
             evs = []
             for l in fused:
                 a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -631,6 +734,7 @@ def main():
             "fused_bn_fwd_cfg4": ["bn_fwd_cfg4", "relu_cfg4:positive_clip_flat_map_f32"],
             "fused_bn_bwd_cfg4": ["bn_bwd_cfg4", "relu_cfg4:positive_clip_flat_map_bwd_f32"],
             "fused_softmax_fwd_cfg3b": ["softmax_cfg3b:softmax_nd_packed_f32", "softmax_cfg3b:softmax_nd_cat_nll_packed_f32"],
+            "fused_softmax_cfg3a": ["softmax_cfg3a"],
         }
         sym_time = {f"{l.group}:{l.symbol.replace('anode_gpu_', '')}": t for l, t in zip(launches, med)}
         for k, (b, s_) in fg.items():
@@ -641,7 +745,17 @@ def main():
                 abi_s = sum(abi_time[p_] if p_ in abi_time else sym_time[p_] for p_ in parts)
                 entry["abi_sequence_us"] = round(abi_s * 1e6, 1)
                 entry["speedup_vs_abi_sequence"] = round(abi_s / s_, 2)
+            entry["launches"] = [{"symbol": l.symbol.replace("anode_gpu_", ""), "us": round(sorted(t)[len(t) // 2] * 1e6, 1)}
+                                 for l, t in zip(fused, ftimes) if l.group == k]
             fused_model[k] = entry
+        if "fused_cast_cfg1" in fused_model:
+            fused_model["fused_cast_cfg1"]["note"] = ("what config 1 names beyond the reference's casts: u8 -> f32 with "
+                                                      "per-channel normalisation in one pass, then f32 -> u8 quantisation; "
+                                                      "quantize is parity unpinned by the reference (it has no such kernel)")
+        for k in ("affine_bn_fwd_cfg2a", "affine_bn_fwd_cfg2b"):
+            if k in fused_model:
+                fused_model[k]["note"] = ("config 2's gamma ~ U(0.5,1.5), beta ~ N(0,0.1), momentum 0.1: single-pass "
+                                          "statistics, normalise + affine, online_average of mean and var (C elements each)")
 
     out = {
         "metric": "achieved HBM GB/s & % of peak: BN fwd/bwd, softmax-NLL, quantize/cast",
@@ -655,17 +769,22 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic",
+        "data": "synthetic: numpy.random.default_rng(0), drawn in float64 and cast to float32, labels from integers()",
         "config": {
             "workload": "configs[1..4], ABI byte model: cast+dequantize u8[256,3,224,224]; BN fwd(3)+bwd(6 launches) "
                         "f32 [256,64,112,112], [256,2048,7,7], [2,32,128,128,128] + ReLU fwd/bwd; softmax+NLL+bwd "
                         "[256,1000] and [8,19,512,1024]",
             "launches_per_step": len(launches),
             "alg_bytes_per_step": step_bytes,
+            "inputs": "one generator, in this order: cfg1 codes integers(0,256), N(0,1) tensor to quantise; cfg2a then "
+                      "cfg2b x = 2 + 3 N(0,1), dy = N(0,1), gamma = U(0.5,1.5), beta = N(0,0.1); cfg3a logits = 2 N(0,1) "
+                      "(variance 4), labels integers(0,1000); cfg3b logits N(0,1), labels integers(0,19) with "
+                      "random() < 0.05 set to 255, dy = 1; cfg4 x = N(0,1), dy = N(0,1), gamma = 1, beta = 0; eps 1e-5",
         },
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "gelem_per_s": round(step_elems / step_s / 1e9, 2),
         "roofline": roofline,
+        "traffic_by_kernel": traffic_by_kernel,
         "breakdown": breakdown,
         "fused_model": fused_model,
         "per_symbol": per_symbol,
@@ -677,7 +796,7 @@ def main():
         except Exception as e:  # noqa: BLE001
             out["graph_replay"] = {"error": repr(e)}
         try:
-            out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches))
+            out["small_shapes"] = small_shape_latency(torch, gpu, small_shape_groups(torch, launches, fused))
         except Exception as e:  # noqa: BLE001
             out["small_shapes"] = {"error": repr(e)}
     if not args.no_cpu_baseline:
