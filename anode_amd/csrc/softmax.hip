@@ -26,13 +26,16 @@ constexpr float kNegInf = -__builtin_huge_valf();
 // row softmax
 // ---------------------------------------------------------------------------
 
-// Optional fused label gather of the row kernels (cat == nullptr: none).  The thread that has just stored the
-// label's probability p also writes nll = -log(p), the value the separate gather would read back and compute; a
-// label >= K gives NaN (or 0 with `ignore`), written by the thread that holds class 0.
+// Optional fused label gather, and optional fused backward, of the row kernels (cat == nullptr: none).  The thread
+// that has just stored probability p of class k also writes what the separate kernels would compute from the stored
+// value: nll = -log(p) if k is the row's label (a label >= K gives NaN, or 0 with `ignore`, written by the thread
+// that holds class 0), and, when dy is given, dx[k] = dy[row] * (p - float(label == k)) (softmax.cu:188-193).
 struct RowNll {
   const uint32_t *cat;
   float *nll;
   bool ignore;
+  const float *dy;  // with dx: the upstream gradient per row, known before the forward pass (e.g. ones for a summed loss)
+  float *dx;
   __device__ bool on() const { return cat != nullptr; }
   __device__ uint32_t label(uint64_t r) const { return cat[r]; }
   // called by the thread that holds class k of row r, with the stored probability
@@ -42,6 +45,7 @@ struct RowNll {
     } else if (k == 0 && label >= K) {
       nll[r] = ignore ? 0.0f : __builtin_nanf("");
     }
+    if (dx != nullptr) dx[size_t(r) * K + k] = dy[r] * (prob - float(label == k));
   }
 };
 
@@ -134,7 +138,14 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
       if (nl.on()) {
         const uint64_t r = r0 + threadIdx.x;
         const uint32_t label = nl.label(r);
-        nl.emit(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
+        if (nl.dx != nullptr) {
+#pragma unroll
+          for (int k = 0; k < KMAX; ++k) {
+            if (uint32_t(k) < K) nl.emit(r, K, label, uint32_t(k), row[k]);
+          }
+        } else {
+          nl.emit(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
+        }
       }
     }
     __syncthreads();
@@ -336,7 +347,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
 }
 
 void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float *x, float *y,
-                         CUstream_st *stream, RowNll nl = RowNll{nullptr, nullptr, false}) {
+                         CUstream_st *stream, RowNll nl = RowNll{nullptr, nullptr, false, nullptr, nullptr}) {
   (void)checked_len(K, R, 1, symbol);
   if (K == 0 || R == 0) return;
   hipStream_t s = as_stream(stream);
@@ -917,7 +928,18 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32(uint32_
 ANODE_EXPORT void anode_gpu_softmax_cat_nll_fused_packed_f32(uint32_t dim0, uint32_t dim1, const float *x,
                                                              const uint32_t *cat_data, float *softmax, float *nll,
                                                              const KernelConfig *, CUstream_st *stream) {
-  launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false});
+  launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
+}
+
+// Additive: the same with the backward of the NLL as well, for callers that know the upstream gradient dy before the
+// forward pass (a summed or averaged loss): dx = dy * (softmax - onehot), the values of
+// anode_gpu_softmax_cat_nll_bwd_packed_f32, from the same launch.  A [256,1000] head is launch-bound: one launch
+// instead of three.
+ANODE_EXPORT void anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *x,
+                                                                     const uint32_t *cat_data, const float *dy,
+                                                                     float *softmax, float *nll, float *dx,
+                                                                     const KernelConfig *, CUstream_st *stream) {
+  launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
 }
 
 // Additive (no counterpart in the reference): softmax_nd and softmax_nd_cat_nll in one pass over x.
@@ -929,7 +951,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
   const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
-    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false});
+    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
   } else if (dim0 <= 32) {
     hipStream_t s = as_stream(stream);
     const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) && aligned16(nll);

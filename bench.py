@@ -248,6 +248,10 @@ def build_workload(torch, only, copy_calibration=False):
         fused.append(Launch("fused_softmax_cfg3a", "anode_gpu_softmax_cat_nll_bwd_packed_f32", (K, R, dy, p2, lab, dx2),
                             8 * K * R + 8 * R, K * R))
 
+        p3, nll3, dx3 = empty(K * R), empty(R), empty(K * R)
+        fused.append(Launch("fused_softmax_fwd_bwd_cfg3a", "anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32",
+                            (K, R, x, lab, dy, p3, nll3, dx3), 12 * K * R + 12 * R, K * R))
+
     # ---- config 3b: channel-axis softmax + NLL [8,19,512,1024] -------------------
     if sm3b is not None:
         P, C, N = 512 * 1024, 19, 8
@@ -508,6 +512,9 @@ def small_shape_groups(torch, launches, fused=()):
     cfg3a_fused = [l for l in fused if l.group == "fused_softmax_cfg3a"]
     if cfg3a_fused:
         groups["softmax_nll_cfg3a_fused_fwd"] = cfg3a_fused  # softmax + NLL in one launch, then the backward
+    one = [l for l in fused if l.group == "fused_softmax_fwd_bwd_cfg3a"]
+    if one:
+        groups["softmax_nll_cfg3a_one_launch"] = one         # softmax + NLL + backward in one launch
     return groups
 
 
@@ -735,6 +742,7 @@ def main():
             "fused_bn_bwd_cfg4": ["bn_bwd_cfg4", "relu_cfg4:positive_clip_flat_map_bwd_f32"],
             "fused_softmax_fwd_cfg3b": ["softmax_cfg3b:softmax_nd_packed_f32", "softmax_cfg3b:softmax_nd_cat_nll_packed_f32"],
             "fused_softmax_cfg3a": ["softmax_cfg3a"],
+            "fused_softmax_fwd_bwd_cfg3a": ["softmax_cfg3a"],
         }
         sym_time = {f"{l.group}:{l.symbol.replace('anode_gpu_', '')}": t for l, t in zip(launches, med)}
         for k, (b, s_) in fg.items():

@@ -240,6 +240,9 @@ void anode_gpu_batch_norm_bwd_apply_3d1_packed_accumulate_f32(uint32_t dim0, uin
 /* Row softmax and softmax_cat_nll in one pass over x (src/ops.rs:1172-1176 as one launch); writes the same softmax and
  * nll as anode_gpu_softmax_packed_*_f32 followed by anode_gpu_softmax_cat_nll_packed_f32 (NaN for a label >= dim0). */
 void anode_gpu_softmax_cat_nll_fused_packed_f32(uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, float *softmax, float *nll, ANODE_LAUNCH_TAIL);
+/* The same plus anode_gpu_softmax_cat_nll_bwd_packed_f32 in that launch, for a dy that is known before the forward
+ * pass (e.g. ones for a summed loss): dx[k,i] = dy[i] * (softmax[k,i] - float(label[i]==k)). */
+void anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, const float *dy, float *softmax, float *nll, float *dx, ANODE_LAUNCH_TAIL);
 /* softmax_nd and softmax_nd_cat_nll in one pass over x; writes the same softmax and nll as the two entry points. */
 void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, float *softmax, float *nll, ANODE_LAUNCH_TAIL);
 /* Running statistics: y <- fma(rate, x - y, y) (the semantics of anode's online_average, tests/test_gpu.rs:561-593). */

@@ -212,6 +212,16 @@ def test_fused_softmax_nll_rows_equals_the_two_launches(oracle, K, R):
         assert_bit_exact(host(nll2), host(nll1), f"fused row nll K={K}")
         assert np.array_equal(np.isnan(host(nll2)), lab >= K)
         assert_close(host(nll2), oracle.softmax_cat_nll(K, R, host(p2), lab, f64=True), "fused nll vs fp64", abs_floor=1e-6)
+        # forward and backward in one launch
+        dy = g.standard_normal(R).astype(F32)
+        dx1 = empty(K * R, offset=offset)
+        call("anode_gpu_softmax_cat_nll_bwd_packed_f32", K, R, dev(dy, offset), p1, dev(lab, offset), dx1)
+        p4, nll4, dx4 = empty(K * R, offset=offset), empty(R, offset=offset), empty(K * R, offset=offset)
+        call("anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32", K, R, dev(x, offset), dev(lab, offset), dev(dy, offset),
+             p4, nll4, dx4)
+        assert_bit_exact(host(p4), host(p1), "fwd+bwd fused softmax")
+        assert_bit_exact(host(nll4), host(nll1), "fwd+bwd fused nll")
+        assert_bit_exact(host(dx4), host(dx1), "fwd+bwd fused dx")
         # the channel-axis entry point with one pixel per sample is the same thing
         p3, nll3 = empty(K * R, offset=offset), empty(R, offset=offset)
         call("anode_gpu_softmax_nd_cat_nll_fused_packed_f32", 1, K, R, dev(x, offset), dev(lab, offset), p3, nll3)
