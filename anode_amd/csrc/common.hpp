@@ -23,6 +23,7 @@ struct CUstream_st;
 namespace anode {
 
 constexpr int kWave = 64;    // CDNA wavefront width
+constexpr uint32_t kXcds = 8;  // accelerator dies of an MI355X; workgroup i of a launch runs on die i % 8
 constexpr int kBlock = 256;  // workgroup size of every kernel here: 4 waves, one per SIMD
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));

@@ -148,7 +148,8 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
     p.vec = (ptrs_aligned && S % 4 == 0) ? 1 : 0;
     if (uint64_t(S) >= 2 * per_tile) {
       p.n_stiles = ceil_div_u32(S, per_tile);
-      p.SB = (ceil_div_u32(S, p.n_stiles) + 3u) & ~3u;
+      // whole 128-byte lines per tile, so that neighbouring tiles (on different XCDs) never fetch the same line
+      p.SB = (ceil_div_u32(S, p.n_stiles) + 31u) & ~31u;
       p.n_stiles = ceil_div_u32(S, p.SB);
       p.NB = 1;
     } else {

@@ -58,7 +58,17 @@ class Launch:
 # of the profile named in TRAFFIC_SOURCE, not re-measured by this run; a launch that is not listed reports null.
 TRAFFIC_SOURCE = "profiles/bench_step_dominant_kernels_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not re-measured in this run)"
 MEASURED_TRAFFIC = {
-    # (symbol, group): bytes
+    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2a"): 2466145290,
+    ("anode_gpu_batch_norm_3d1_packed_f32", "bn_fwd_cfg2a"): 1644145154,
+    ("anode_gpu_batch_mean_3d1_packed_f32", "bn_fwd_cfg2b"): 102822715,
+    ("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", "bn_bwd_cfg2b"): 205590138,
+    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): 308432498,
+    ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): 1610539015,
+    ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): 637599226,
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): 291540413,
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): 671085056,
+    ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): 192705077,
+    ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): 192703030,
 }
 
 
@@ -303,6 +313,25 @@ def stream_probe(torch, gpu):
             lambda i: gpu.call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, pairs[i % 4][0], mean), 4 * n)
     for k, v in enumerate(saved):
         gpu.set_tuning(k, v)
+    del pairs
+    torch.cuda.empty_cache()
+
+    # What a plane-strided walk costs at config 3b, [8,19,512,1024] (319 MB arrays), library defaults: a flat copy,
+    # the n-d NLL backward (reads one plane and writes one plane at a time: no dependency between planes), and the n-d
+    # softmax (all 19 planes of a pixel group must have arrived before the first can be stored), each from cold arrays.
+    P, Cc, Nn = 512 * 1024, 19, 8
+    m = P * Cc * Nn
+    sets = [(torch.randn(m, device="cuda"), torch.empty(m, device="cuda")) for _ in range(3)]
+    lab = torch.randint(0, Cc, (P * Nn,), device="cuda", dtype=torch.int32)
+    ones = torch.ones(P * Nn, device="cuda")
+    out["planes_319MB_gbps"] = {
+        "flat_copy": rate(lambda i: gpu.call("anode_gpu_copy_flat_map_f32", m, *sets[i % 3]), 8 * m),
+        "softmax_nd_cat_nll_bwd (plane by plane)": rate(
+            lambda i: gpu.call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, Cc, Nn, ones, sets[i % 3][0], lab,
+                               sets[i % 3][1]), 8 * m + 8 * P * Nn),
+        "softmax_nd (all planes, then store)": rate(
+            lambda i: gpu.call("anode_gpu_softmax_nd_packed_f32", P, Cc, Nn, *sets[i % 3]), 8 * m),
+    }
     return out
 
 
@@ -353,7 +382,7 @@ def all_symbols(torch, gpu):
     # flat maps and the join on the same 822 MB arrays
     fl = f"[{n}]"
     for name in ("copy", "modulus", "square", "sqrt", "positive_clip", "logistic", "unit_step", "normal_cdf", "tanh",
-                 "rcosh2"):
+                 "rcosh2", "log_positive_clip", "positive_reciprocal"):
         add(f"anode_gpu_{name}_flat_map_f32", fl, (n, x, y), 8 * n)
     add("anode_gpu_leaky_relu_flat_map_f32", fl, (n, 0.1, x, y), 8 * n)
     add("anode_gpu_positive_clip_flat_map_bwd_f32", fl, (n, dy, x, y), 12 * n)
@@ -384,6 +413,9 @@ def all_symbols(torch, gpu):
             add("anode_gpu_softmax_cat_nll_bwd_packed_f32", rs, (K, R, dy, x, lab, y), 8 * K * R + 8 * R)
             add("anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32", rs, (K, R, dy, x, lab, dx), 12 * K * R + 8 * R)
             add("anode_gpu_arg_max_packed_u32", rs, (K, R, x, E(R, torch.int32)), 4 * K * R + 4 * R)
+            add("anode_gpu_softmax_cat_nll_fused_packed_f32", rs, (K, R, x, lab, y, E(R)), 8 * K * R + 8 * R)
+            add("anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32", rs, (K, R, x, lab, dy, y, E(R), dx),
+                12 * K * R + 12 * R)
 
     # channel-axis softmax / NLL / one-hot / F1 on [8,19,512,1024]
     P, Cc, Nn = 512 * 1024, 19, 8
