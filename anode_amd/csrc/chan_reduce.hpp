@@ -73,17 +73,6 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
 //     (NIN == 3: term3(const Param&, float a, float b, float c, double &s0, double &s1, double &s2))
 //   __device__ void finalize(uint32_t c, double s0, double s1, double s2) const;   // writes the output(s)
 
-// Neighbouring channel tiles share a 128-byte line wherever a tile's run is not a whole number of lines (196 * CB
-// bytes at S = 49).  Workgroups go to the 8 XCDs in turn, each with an L2 of its own, so tiles are dealt in
-// contiguous ranges per XCD: tile index i of n becomes the (i / 8)-th tile of the range of XCD i % 8.  The
-// neighbour's half of a shared line is then an L2 hit instead of a second fetch from memory (FETCH_SIZE 1.14 x the
-// array -> 1.00 x, 21.9 -> 20.3 us, for batch_mean at [49, 2048, 256]).
-__device__ inline uint32_t xcd_contiguous(uint32_t i, uint32_t n) {
-  const uint32_t xcd = i % kXcds, turn = i / kXcds;
-  const uint32_t per = n / kXcds, rem = n % kXcds;
-  return xcd * per + min(xcd, rem) + turn;
-}
-
 template <typename Op, typename P>
 __device__ inline void chan_reduce_term(const Op &op, const P &prm, float a, float b, float c, double &s0,
                                         double &s1, double &s2) {

@@ -94,6 +94,20 @@ inline void with_stream_policy(int nt, F &&f) {
   }
 }
 
+// Workgroups go to the 8 XCDs in turn, each with an L2 (and address translation cache) of its own.  Dealing tiles in
+// contiguous ranges per XCD -- tile index i of n becomes the (i / 8)-th tile of the range of XCD i % 8 -- keeps
+// neighbouring tiles on one XCD.  Where neighbours share 128-byte lines (a tile's run is not a whole number of
+// lines: 196 * CB bytes at S = 49) the neighbour's half of a line is then an L2 hit instead of a second fetch from
+// memory (FETCH_SIZE 1.14 x the array -> 1.00 x, 21.9 -> 20.3 us, for batch_mean at [49, 2048, 256]).  Of the
+// plane-strided n-d kernels the NLL backward gains 4 % inside a softmax + NLL + backward sequence (106 -> 102 us at
+// [512K, 19, 8]) while the softmax itself loses 7 % there (it gains 3 % run alone), so only the backward uses it;
+// flat maps gain nothing.
+__device__ inline uint32_t xcd_contiguous(uint32_t i, uint32_t n) {
+  const uint32_t xcd = i % kXcds, turn = i / kXcds;
+  const uint32_t per = n / kXcds, rem = n % kXcds;
+  return xcd * per + min(xcd, rem) + turn;
+}
+
 template <int NT, typename V>
 __device__ inline V load_stream(const V *p) {
   if constexpr ((NT & kNtLoad) != 0) {
@@ -226,6 +240,7 @@ struct Tuning {
   Knob reduce_single_pass_grid;  // lane tiles: with at least this many channel groups a tile takes all samples
   Knob reduce_lanes_max_ctiles;  // lane tiles: most channel groups (bounds the grid for very many channels)
   Knob reduce_lanes_min_run;     // lane tiles: fewest contiguous floats a tile reads per sample
+  Knob nd_xcd_mask;              // n-d softmax kernels that deal pixel groups per XCD: 1 softmax, 2 NLL backward (default), 4 NLL gather
 };
 
 // The streaming mask to use for an array of `bytes` bytes: the load bit of `mask` from nt_min_bytes on, the store

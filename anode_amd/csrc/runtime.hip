@@ -377,7 +377,7 @@ ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return a
 // Test and measurement hook (not declared in the public header).  Knobs: 0 flat_wg_per_cu, 2 reduce_wg_target,
 // 3 nontemporal (0, 1 or 3: streaming loads without streaming stores is not a policy the maps are built for),
 // 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes, 8 reduce_tile_pos,
-// 9 reduce_lanes, 10 reduce_single_pass_grid, 11 reduce_lanes_max_ctiles, 12 reduce_lanes_min_run.  Returns the previous value; a
+// 9 reduce_lanes, 10 reduce_single_pass_grid, 11 reduce_lanes_max_ctiles, 12 reduce_lanes_min_run, 13 nd_xcd_mask.  Returns the previous value; a
 // negative value only reads.  Returns -1, and changes nothing, for an unknown knob or a value the knob does not take.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
   anode::Tuning &t = anode::tuning();
@@ -395,6 +395,7 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 10: slot = &t.reduce_single_pass_grid; break;
     case 11: slot = &t.reduce_lanes_max_ctiles; break;
     case 12: slot = &t.reduce_lanes_min_run; break;
+    case 13: slot = &t.nd_xcd_mask; break;
     default: return -1;
   }
   if (knob == 3 && value >= 0 && value != 0 && value != 1 && value != 3) return -1;

@@ -521,6 +521,7 @@ struct PixelGrid {
   uint32_t P, C, N;
   uint32_t total_groups;
   uint32_t ignore;  // 1: an out-of-range label gives nll = 0 and no gradient, instead of NaN and dy * p
+  uint32_t xcd;     // 1: pixel groups are dealt to the XCDs in contiguous ranges (xcd_contiguous)
   FastDiv div_gps;  // groups per sample
 };
 
@@ -554,7 +555,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
   typedef typename PixVec<V>::U U;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   const uint64_t total = uint64_t(pg.total_groups) * SPLIT;
-  for (uint64_t t = uint64_t(blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
+  for (uint64_t t = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
     // the lanes of a pair are neighbours (t even, t + 1), so they always run, and leave the loop, together
     const uint32_t g = uint32_t(t / SPLIT), h = uint32_t(t % SPLIT);
     uint32_t p, n;
@@ -629,7 +630,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
                                                                    float *__restrict__ y) {
   constexpr int W = PixVec<V>::W;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
@@ -654,7 +655,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t pix = size_t(p) + size_t(pg.P) * n;
@@ -686,7 +687,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, g, W, p, n);
     const size_t pix = size_t(p) + size_t(pg.P) * n;
@@ -719,6 +720,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
 PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore = false) {
   PixelGrid pg;
   pg.ignore = ignore ? 1u : 0u;
+  pg.xcd = 0u;
   pg.P = P;
   pg.C = C;
   pg.N = N;
@@ -736,7 +738,8 @@ template <typename V, bool NLL, int NT>
 void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
                               float *nll, hipStream_t s) {
   constexpr int SPLIT = PixVec<V>::W == 4 ? 2 : 1;
-  const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
+  PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
+  pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
   const uint32_t blocks = stream_grid(uint64_t(pg.total_groups) * SPLIT, 1);
   if (C <= 4) {
     softmax_nd_reg_kernel<4, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
@@ -825,7 +828,8 @@ void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint3
   (void)checked_len(P, C, N, symbol);
   if (P == 0 || N == 0) return;
   if (P % 4 == 0 && aligned16(cat) && aligned16(nll)) {
-    const PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
+    PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
+    pg.xcd = (tuning().nd_xcd_mask & 4) ? 1u : 0u;
     softmax_nd_cat_nll_kernel<f32x4><<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, prob, cat, nll);
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, 1, ignore);
@@ -847,7 +851,8 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   if (vec) {
-    const PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
+    PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
+    pg.xcd = (tuning().nd_xcd_mask & 2) ? 1u : 0u;
     with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
       softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, decltype(policy)::value>
           <<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
