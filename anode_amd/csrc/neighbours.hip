@@ -34,6 +34,14 @@ struct OnlineAddMap {
   __device__ float value(const Param &, float a, float, uint32_t) const { return rate * a; }
   __device__ float accum(const Param &, float a, float, uint32_t, float old) const { return fmaf(rate, a, old); }
 };
+// y = fma(rate, y, x): the running value is discounted, then the new one added
+struct OnlineDiscountMap {
+  float rate;
+  typedef NoParam Param;
+  __device__ Param load(uint32_t) const { return Param{}; }
+  __device__ float value(const Param &, float a, float, uint32_t) const { return a; }
+  __device__ float accum(const Param &, float a, float, uint32_t, float old) const { return fmaf(rate, old, a); }
+};
 struct IsNonzeroMap {
   typedef NoParam Param;
   __device__ Param load(uint32_t) const { return Param{}; }
@@ -136,4 +144,9 @@ ANODE_EXPORT void anode_gpu_is_nonzero_packed_f32(uint32_t len, const float *x, 
 ANODE_EXPORT void anode_gpu_online_add_packed_f32(uint32_t len, float rate, const float *x, float *y,
                                                   const KernelConfig *, CUstream_st *stream) {
   launch_chan_map<1, true>(__func__, len, 1, 1, OnlineAddMap{rate}, x, nullptr, y, stream);
+}
+
+ANODE_EXPORT void anode_gpu_online_discount_packed_f32(uint32_t len, float rate, const float *x, float *y,
+                                                       const KernelConfig *, CUstream_st *stream) {
+  launch_chan_map<1, true>(__func__, len, 1, 1, OnlineDiscountMap{rate}, x, nullptr, y, stream);
 }

@@ -286,6 +286,9 @@ void anode_gpu_mult_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAU
 void anode_gpu_is_nonzero_packed_f32(uint32_t len, const float *x, float *y, ANODE_LAUNCH_TAIL);
 /* src/ops_gpu.rs:5886 (online_add): y[i] = fma(rate, x[i], y[i]). */
 void anode_gpu_online_add_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
+/* src/ops_gpu.rs:5972, :6015 (online_discount; the momentum buffer of src/ops.rs:1425-1430): y[i] = fma(rate, y[i], x[i]).
+ * The arithmetic is read off the name and the momentum recipe; gpudevicemem's kernel is not in the reference tree. */
+void anode_gpu_online_discount_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
 
 /* The same five under the link names anode calls them by, directly over FFI, for a build that has no ROCm
  * gpudevicemem yet.  In the static archive they sit in an object of their own (gpudevicemem_names.o), which the

@@ -925,6 +925,11 @@ ORACLE_API void oracle_online_add(uint32_t len, float rate, const float *x, floa
   for (uint32_t i = 0; i < len; ++i) y[i] = fmaf(rate, x[i], y[i]);
 }
 
+/* src/ops_gpu.rs:5972, src/ops.rs:1425-1430: y <- rate * y + x, one fmaf (momentum buffer) */
+ORACLE_API void oracle_online_discount(uint32_t len, float rate, const float *x, float *y) {
+  for (uint32_t i = 0; i < len; ++i) y[i] = fmaf(rate, y[i], x[i]);
+}
+
 /* src/ops_gpu.rs:9592: y[a,b] = x[a,b] / r[b], IEEE division */
 ORACLE_API void oracle_flat_bcast_rdiv(uint32_t inner, uint32_t outer, const float *x, const float *r,
                                        float *y) {

@@ -433,6 +433,13 @@ def sum_packed(x) -> float:
     return float(fn(u32(x.size), _p(x)))
 
 
+def online_discount(rate, x, y):
+    x = _f32(x).ravel()
+    out = _f32(y).ravel().copy()
+    lib().oracle_online_discount(u32(x.size), f32(rate), _p(x), _p(out))
+    return out
+
+
 def online_add(rate, x, y):
     x = _f32(x).ravel()
     out = _f32(y).ravel().copy()

@@ -49,6 +49,10 @@ def test_fill_add_mult_nonzero(n):
         call("anode_gpu_online_add_packed_f32", n, 0.1, dev(x, offset), y)
         with np.errstate(all="ignore"):
             assert_bit_exact(host(y), oracle.online_add(0.1, x, y0), "online_add")
+        y = dev(y0, offset)
+        call("anode_gpu_online_discount_packed_f32", n, 0.9, dev(x, offset), y)
+        with np.errstate(all="ignore"):
+            assert_bit_exact(host(y), oracle.online_discount(0.9, x, y0), "online_discount")
 
 
 @pytest.mark.parametrize("n", LENS)
@@ -192,3 +196,15 @@ def test_nd_nll_ignore(P, C, N):
              dev(lab, offset), dx)
         assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy_masked, p, lab, dx_in=old),
                          "nd bwd ignore accumulate")
+
+
+def test_momentum_step_recipe():
+    # src/ops.rs:1425-1430: buffer <- momentum * buffer + grad, then params <- params + step * buffer
+    buf = dev(np.zeros(1000, F32))
+    grad = dev(np.ones(1000, F32))
+    params = dev(np.full(1000, 3.0, F32))
+    for k in range(1, 4):
+        call("anode_gpu_online_discount_packed_f32", 1000, 0.5, grad, buf)
+        assert np.all(host(buf) == F32(2.0 - 2.0 ** (1 - k)))
+    call("anode_gpu_online_add_packed_f32", 1000, -0.25, buf, params)
+    assert np.all(host(params) == F32(3.0 - 0.25 * 1.75))

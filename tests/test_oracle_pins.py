@@ -90,6 +90,20 @@ def test_ref_online_average_quarter_steps(oracle):
     assert np.all(y == F32(0.4375))
 
 
+def test_online_discount_is_the_geometric_momentum_sum(oracle):
+    # src/ops.rs:1425-1430: the momentum buffer starts at zero and takes y <- rate * y + grad each step.  With a
+    # constant gradient of 1 and rate 1/2 the buffer is 2 - 2^(1-k): exactly representable, so a swapped operand
+    # (rate * x + y gives k/2) or the running-average form (y + rate * (x - y) gives 1 - 2^-k) fails.
+    y = np.zeros(257, F32)
+    for k in range(1, 6):
+        y = oracle.online_discount(0.5, np.ones(257, F32), y)
+        assert np.all(y == F32(2.0 - 2.0 ** (1 - k)))
+    # rate 0 forgets everything, rate 1 is a plain sum
+    x = np.random.default_rng(3).standard_normal(257).astype(F32)
+    assert np.array_equal(oracle.online_discount(0.0, x, y), x)
+    assert np.array_equal(oracle.online_discount(1.0, x, y), (y + x).astype(F32))
+
+
 # --------------------------------------------------------------------------
 # bit-exact class: exact arithmetic and brute force
 # --------------------------------------------------------------------------
