@@ -274,6 +274,10 @@ struct MeanVarReduce {
   float *mean, *var;
   uint32_t S;
   double n, eps;
+  // running statistics updated in the same launch (null: none): y <- fma(rate, stat - y, y), the arithmetic of
+  // online_average applied to the fp32 mean and variance that are stored
+  float *run_mean = nullptr, *run_var = nullptr;
+  float rate = 0.0f;
   __device__ Param load(uint32_t c) const { return double(x[size_t(c) * S]); }
   __device__ void term(const Param &k, float a, float, double &s0, double &s1, double &) const {
     const double d = double(a) - k;
@@ -282,8 +286,12 @@ struct MeanVarReduce {
   }
   __device__ void finalize(uint32_t c, double s0, double s1, double) const {
     const double k = n > 0.0 ? double(x[size_t(c) * S]) : 0.0;  // an empty array has no first element to read
-    mean[c] = float(k + s0 / n);
-    var[c] = float((s1 - s0 * s0 / n) / n + eps);
+    const float m = float(k + s0 / n);
+    const float v = float((s1 - s0 * s0 / n) / n + eps);
+    mean[c] = m;
+    var[c] = v;
+    if (run_mean) run_mean[c] = fmaf(rate, m - run_mean[c], run_mean[c]);
+    if (run_var) run_var[c] = fmaf(rate, v - run_var[c], run_var[c]);
   }
 };
 
@@ -555,6 +563,20 @@ ANODE_EXPORT void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_
                                                           const KernelConfig *, CUstream_st *stream) {
   launch_chan_reduce(__func__, dim0, dim1, dim2,
                      MeanVarReduce{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)}, x, nullptr, stream);
+}
+
+// The same with the layer's running statistics updated by the workgroup that finalises a channel: what
+// src/ops.rs:999-1003 does with batch_mean, batch_var and two online_average launches.
+ANODE_EXPORT void anode_gpu_batch_mean_var_online_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,
+                                                                 float epsilon, float rate, const float *x,
+                                                                 float *mean, float *var, float *run_mean,
+                                                                 float *run_var, const KernelConfig *,
+                                                                 CUstream_st *stream) {
+  MeanVarReduce op{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)};
+  op.run_mean = run_mean;
+  op.run_var = run_var;
+  op.rate = rate;
+  launch_chan_reduce(__func__, dim0, dim1, dim2, op, x, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -231,6 +231,12 @@ def build_workload(torch, only, copy_calibration=False):
                 fused.append(Launch(g_, "anode_gpu_batch_norm_affine_3d1_packed_f32", (*d, x, m2, v2, gamma, beta, y2), 8 * n, n))
                 fused.append(Launch(g_, "anode_gpu_online_average_packed_f32", (C, 0.1, m2, rm), 12 * C, C))
                 fused.append(Launch(g_, "anode_gpu_online_average_packed_f32", (C, 0.1, v2, rv), 12 * C, C))
+                # the same layer with the running statistics moved by the statistics launch itself
+                rm2, rv2 = torch.zeros(C, device="cuda"), torch.ones(C, device="cuda")
+                g2_ = f"affine_one_stats_launch_{f}"
+                fused.append(Launch(g2_, "anode_gpu_batch_mean_var_online_3d1_packed_f32",
+                                    (*d, 1e-5, 0.1, x, m2, v2, rm2, rv2), 4 * n + 24 * C, n))
+                fused.append(Launch(g2_, "anode_gpu_batch_norm_affine_3d1_packed_f32", (*d, x, m2, v2, gamma, beta, y2), 8 * n, n))
         return x, dy, y, dx
 
     bn("cfg2a")
@@ -373,6 +379,7 @@ def all_symbols(torch, gpu):
     add("anode_gpu_batch_mean_bwd_3d1_packed_accumulate_f32", sh, (*d, dm, dx), 8 * n)
     # additive batch-norm entry points on the same arrays
     add("anode_gpu_batch_mean_var_3d1_packed_f32", sh, (*d, 1e-5, x, E(C), E(C)), 4 * n)
+    add("anode_gpu_batch_mean_var_online_3d1_packed_f32", sh, (*d, 1e-5, 0.1, x, E(C), E(C), Rn(C), Rn(C)), 4 * n)
     add("anode_gpu_batch_norm_positive_clip_3d1_packed_f32", sh, (*d, x, m, v, y), 8 * n)
     add("anode_gpu_batch_norm_affine_3d1_packed_f32", sh, (*d, x, m, v, dm, dv, y), 8 * n)
     add("anode_gpu_batch_norm_bwd_reduce_3d1_packed_f32", sh, (*d, dy, x, m, v, None, E(C), E(C)), 8 * n)
@@ -850,6 +857,10 @@ def main():
             if k in fused_model:
                 fused_model[k]["note"] = ("config 2's gamma ~ U(0.5,1.5), beta ~ N(0,0.1), momentum 0.1: single-pass "
                                           "statistics, normalise + affine, online_average of mean and var (C elements each)")
+        for k in ("affine_one_stats_launch_bn_fwd_cfg2a", "affine_one_stats_launch_bn_fwd_cfg2b"):
+            if k in fused_model:
+                fused_model[k]["note"] = ("the same layer in two launches: the statistics launch also moves the running "
+                                          "mean and variance (bit-identical to the four launches of affine_bn_fwd_*)")
 
     out = {
         "metric": "achieved HBM GB/s & % of peak: BN fwd/bwd, softmax-NLL, quantize/cast",

@@ -215,6 +215,11 @@ void anode_gpu_quantize_u8_packed_f32(uint32_t len, float lo, float hi, const fl
 void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32_t inner_dim, uint32_t bcast_dim, uint32_t outer_dim, const float *scale, const float *shift, const uint8_t *x, float *y, ANODE_LAUNCH_TAIL);
 /* batch_mean and batch_var in one pass over x: mean[c], var[c] = biased variance + epsilon (composes with batch_norm). */
 void anode_gpu_batch_mean_var_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, float *mean, float *var, ANODE_LAUNCH_TAIL);
+/* The same launch also moves the layer's running statistics (src/ops.rs:1002-1003: online_average of the mean and of
+ * var + epsilon): run[c] = fma(rate, stat[c] - run[c], run[c]) on the fp32 values stored in mean and var, so the
+ * result equals batch_mean_var followed by two anode_gpu_online_average_packed_f32 launches bit for bit.  Either
+ * running array may be null. */
+void anode_gpu_batch_mean_var_online_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, float rate, const float *x, float *mean, float *var, float *run_mean, float *run_var, ANODE_LAUNCH_TAIL);
 /* batch_mean_var for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  No counterpart in the reference (whose one-block-per-channel reductions need no
  * workspace).  Same kernels, geometry and results as anode_gpu_batch_mean_var_3d1_packed_f32, but the partial sums

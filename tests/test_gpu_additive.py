@@ -103,6 +103,19 @@ def test_channel_sums_and_mean_var(oracle, S, C, N):
         call("anode_gpu_batch_var_3d1_packed_f32", S, C, N, 1e-5, xd, m2, v2)
         assert_bit_exact(host(mean), host(m2), "mean: one pass vs two")
         assert_close(host(var), host(v2), "var: one pass vs two")
+        # with the running statistics moved in the same launch: the bits of mean_var followed by two online_average
+        g2 = np.random.default_rng(C)
+        rm0, rv0 = g2.standard_normal(C).astype(F32), g2.uniform(0.5, 2.0, C).astype(F32)
+        rm1, rv1 = dev(rm0, offset), dev(rv0, offset)
+        call("anode_gpu_online_average_packed_f32", C, 0.1, mean, rm1)
+        call("anode_gpu_online_average_packed_f32", C, 0.1, var, rv1)
+        m3, v3, rm2, rv2 = empty(C, offset=offset), empty(C, offset=offset), dev(rm0, offset), dev(rv0, offset)
+        call("anode_gpu_batch_mean_var_online_3d1_packed_f32", S, C, N, 1e-5, 0.1, xd, m3, v3, rm2, rv2)
+        assert_bit_exact(host(m3), host(mean), "mean_var_online mean")
+        assert_bit_exact(host(v3), host(var), "mean_var_online var")
+        assert_bit_exact(host(rm2), host(rm1), "running mean")
+        assert_bit_exact(host(rv2), host(rv1), "running var")
+        assert_bit_exact(host(rm2), oracle.online_average(0.1, host(mean), rm0), "running mean vs oracle")
     xs = x[:S * C]
     y = empty(C)
     call("anode_gpu_sum_Iab_Ob_packed_deterministic_f32", S, C, dev(xs), y)
@@ -239,6 +252,20 @@ def test_ref_fused_softmax_nll_known_answers():
     call("anode_gpu_softmax_cat_nll_fused_packed_f32", 32, 2, dev(np.zeros(64, F32)), dev(np.array([12, 42], np.uint32)), p, nll)
     h = host(nll)
     assert np.isfinite(h[0]) and np.isnan(h[1]) and np.isnan(h.sum())
+
+
+def test_running_statistics_in_the_statistics_launch_known_answers():
+    # x == 3 everywhere: mean 3, variance 0 + eps; from running values 1 and 1 at rate 1/4 (the arithmetic of
+    # tests/test_gpu.rs:561-593): 1 + (3 - 1)/4 = 1.5 and 1 + (eps - 1)/4; null running arrays are skipped
+    S, C, N = 49, 8, 4
+    x = dev(np.full(S * C * N, 3.0, F32))
+    m, v, rm, rv = empty(C), empty(C), dev(np.ones(C, F32)), dev(np.ones(C, F32))
+    call("anode_gpu_batch_mean_var_online_3d1_packed_f32", S, C, N, 0.5, 0.25, x, m, v, rm, rv)
+    assert np.all(host(m) == F32(3.0)) and np.all(host(v) == F32(0.5))
+    assert np.all(host(rm) == F32(1.5)) and np.all(host(rv) == F32(0.875))
+    m2, v2 = empty(C), empty(C)
+    call("anode_gpu_batch_mean_var_online_3d1_packed_f32", S, C, N, 0.5, 0.25, x, m2, v2, None, None)
+    assert np.all(host(m2) == F32(3.0)) and np.all(host(v2) == F32(0.5))
 
 
 def test_ref_online_average_quarter_steps(oracle):
