@@ -154,7 +154,7 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t 
   for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
     const uint32_t w = x4[g];
     uint32_t q, s;
-    div_s.divmod(g * 4u, q, s);
+    div_s.divmod(uint32_t(g) * 4u, q, s);  // 4 g < len, which fits 32 bits
     uint32_t c = q - div_c.div(q) * C;
     float a = scale[c], b = shift[c];
     f32x4 r;
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8_scalar_kernel(uint
                                                                             float *__restrict__ y) {
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) {
-    const uint32_t q = div_s.div(i);
+    const uint32_t q = div_s.div(uint32_t(i));  // i < len, which fits 32 bits
     const uint32_t c = q - div_c.div(q) * div_c.d;
     y[i] = fmaf(scale[c], float(x[i]), shift[c]);
   }

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(kBlock) void one_hot_kernel(uint32_t P, uint32_t K,
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < total_groups; g += stride) {
     uint32_t n, r;
-    div_gps.divmod(g, n, r);
+    div_gps.divmod(uint32_t(g), n, r);  // g < total_groups, which fits 32 bits
     const uint32_t p = r * uint32_t(W);
     const U lab = *reinterpret_cast<const U *>(cat + (size_t(p) + size_t(P) * n));
     const size_t base = size_t(p) + size_t(P) * K * n;

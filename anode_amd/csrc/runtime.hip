@@ -40,6 +40,7 @@ Tuning g_tuning = {
     /*reduce_single_pass_grid=*/{{256}},
     /*reduce_lanes_max_ctiles=*/{{2048}},
     /*reduce_lanes_min_run=*/{{128}},
+    /*nd_xcd_mask=*/{{2}},
     };
 
 }  // namespace

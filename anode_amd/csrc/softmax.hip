@@ -559,7 +559,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     // the lanes of a pair are neighbours (t even, t + 1), so they always run, and leave the loop, together
     const uint32_t g = uint32_t(t / SPLIT), h = uint32_t(t % SPLIT);
     uint32_t p, n;
-    pixel_decode(pg, g, W, p, n);
+    pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     V v[H];
 #pragma unroll
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
-    pixel_decode(pg, g, W, p, n);
+    pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     V m = PixVec<V>::splat(kNegInf);
     for (uint32_t k = 0; k < pg.C; ++k) m = vmax(m, *reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
@@ -657,7 +657,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
-    pixel_decode(pg, g, W, p, n);
+    pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     const U lab = *reinterpret_cast<const U *>(cat + pix);
@@ -689,7 +689,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
-    pixel_decode(pg, g, W, p, n);
+    pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     V d = *reinterpret_cast<const V *>(dy + pix);
