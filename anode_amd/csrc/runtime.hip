@@ -168,7 +168,10 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
     // a tile that is not the whole channel axis must start on a 16-byte boundary: CB*S a multiple of 4
     const uint32_t unit = 4 / gcd_u32(S, 4);
     const uint32_t lane_cap = kBlock * (vec ? 4u : 1u);  // positions that one pass of a workgroup's lanes covers
-    bool lanes = g_tuning.reduce_lanes > 0 && S <= lane_cap && (!vec || C <= unit || unit * S <= lane_cap);
+    // (with 16-byte accesses a tile is either the whole channel axis or a multiple of `unit` channels: one of the
+    // two must fit the lanes)
+    bool lanes = g_tuning.reduce_lanes > 0 && S <= lane_cap &&
+                 (!vec || uint64_t(C) * S <= lane_cap || uint64_t(unit) * S <= lane_cap);
     if (lanes) {
       // "lane" tiles: few channels, all (or many) samples, several samples side by side in the workgroup
       uint32_t cb_max = lane_cap / S;

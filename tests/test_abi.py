@@ -271,6 +271,7 @@ PLAN_SHAPES = [
     (784, 16, 32), (12544, 64, 256), (49, 2048, 256), (2097152, 32, 2), (1, 1000, 64), (1, 1, 1), (3, 5, 7),
     (4097, 3, 9), (4096, 1, 1), (50, 3, 2), (12321, 8, 4), (7, 300000, 2), (100000, 4, 1), (1024, 3, 4), (1023, 7, 4),
     (1025, 5, 3), (196, 512, 64), (300, 64, 32), (2, 3, 1000), (1, 65536, 4096), (255, 9, 2), (257, 9, 2),
+    (465, 4, 1),   # 16-byte accesses, C no larger than the channel unit, C*S beyond one pass of the lanes
 ]
 
 
@@ -312,6 +313,27 @@ def test_reduction_tiling_covers_the_array_exactly_once(S, C, N):
             assert not p["vec"]
 
 
+def test_reduction_tiling_on_drawn_shapes():
+    # every branch of the planner on shapes nobody picked: S, C, N log-uniform, both alignments, one and two inputs
+    # (a planner bug shows as a failed invariant here, or as a crash of this process: it is host arithmetic)
+    g = np.random.default_rng(2024)
+
+    def draw(lo, hi):
+        return max(lo, min(hi, int(round(float(np.exp(g.uniform(np.log(lo), np.log(hi + 1))))))))
+
+    done = 0
+    while done < 4000:
+        S, C, N = draw(1, 3000000), draw(1, 70000), draw(1, 5000)
+        if S * C * N >= 2 ** 32:
+            continue
+        done += 1
+        for flags in (0, 1, 2, 3):
+            out = (ctypes.c_uint32 * 12)()
+            _lib.load().cdll.anode_gpu_plan_reduce(S, C, N, flags, out)
+            keys = ["whole", "CB", "SB", "n_ctiles", "n_stiles", "NB", "n_ntiles", "ppc", "vec", "grid", "P", "J"]
+            _check_plan(dict(zip(keys, list(out))), S, C, N, bool(flags & 1))
+
+
 def test_reduction_tiling_without_lane_tiles():
     # tuning knob 9 = 0 switches lane tiles off: short channels then use the wide tiles (in a child process, so that
     # the knob does not leak into other tests)
@@ -337,6 +359,55 @@ print(json.dumps(out))
         p = dict(zip(keys, v))
         assert p["whole"] != 2
         _check_plan(p, S, C, N, bool(al))
+
+
+_HOST_SWEEP = r"""
+import ctypes, sys
+sys.path.insert(0, {root!r})
+import numpy as np
+from anode_amd import _lib
+from anode_amd._lib import KernelConfig
+lib = _lib.load()
+cfg = KernelConfig(1024, 1024)
+g = np.random.default_rng(5)
+def draw(hi):
+    return max(1, min(hi, int(round(float(np.exp(g.uniform(0.0, np.log(hi + 1))))))))
+calls = 0
+for name, (restype, argtypes, pnames) in sorted(lib.prototypes.items()):
+    if pnames[-2:] != ["cfg", "stream"]:
+        continue
+    fn = lib.symbol(name)
+    n_dims = sum(1 for t in argtypes[:-2] if t is ctypes.c_uint32)
+    for it in range(40):
+        while True:
+            dims = [0 if g.random() < 0.03 else draw((3000000, 70000, 5000, 100)[min(k, 3)]) for k in range(n_dims)]
+            if np.prod([max(d, 1) for d in dims], dtype=object) < 2 ** 32:
+                break
+        skew = 0 if g.random() < 0.7 else 4      # 16-byte aligned or element-aligned pointers (never dereferenced)
+        args, k = [], 0
+        for i, t in enumerate(argtypes[:-2]):
+            if t is ctypes.c_uint32:
+                args.append(dims[k]); k += 1
+            elif t is ctypes.c_void_p:
+                args.append(0x7f0000001000 + skew + 0x100000 * i)
+            else:
+                args.append(float(g.uniform(0.01, 2.0)))
+        fn(*args, ctypes.byref(cfg), None)
+        lib.symbol("anode_gpu_take_last_error")()
+        calls += 1
+print("calls", calls)
+"""
+
+
+def test_host_side_of_every_entry_point_survives_drawn_shapes():
+    # With no device visible every launch fails and is recorded, so what runs is the host arithmetic of each entry
+    # point (tiling plans, grids, exact-division constants) on drawn dims and alignments: it must neither trap nor
+    # abort.  (A planner once divided by zero at [465, 4, 1].)
+    env = dict(os.environ, HIP_VISIBLE_DEVICES="", ROCR_VISIBLE_DEVICES="")
+    r = subprocess.run([sys.executable, "-c", _HOST_SWEEP.format(root=_lib.REPO_ROOT)], capture_output=True, text=True,
+                       timeout=600, env=env)
+    assert r.returncode == 0, (r.returncode, r.stdout[-500:], r.stderr[-2000:])
+    assert int(r.stdout.split()[-1]) >= 40 * 90
 
 
 def test_tuning_defaults():

@@ -23,6 +23,8 @@ SHAPES = [
     (16, 300, 3),     # more channels than a tile may hold
     (7, 513, 2),
     (3000, 2, 2),     # one channel per tile, below the chunk threshold
+    (465, 4, 1),      # 16-byte accesses, C*S beyond one pass of a workgroup's lanes, C within the channel unit
+    (465, 4, 3),
     (4096, 2, 3),
     (5000, 3, 4),     # chunk tiles, several samples per tile
     (5001, 2, 3),     # chunk tiles, S odd: element path

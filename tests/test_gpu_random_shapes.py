@@ -7,6 +7,8 @@ too.  Every output lies between two guard bands that must come back untouched:
 a store that strays outside its array fails here even where it lands in memory
 the process owns.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -16,6 +18,7 @@ from gpu_util import F32, assert_bit_exact, assert_close, call, dev, host, rms
 pytestmark = pytest.mark.gpu
 
 GUARD = 64  # elements on either side of an output
+SCALE = max(1, int(os.environ.get("ANODE_DRAWN_CASES_SCALE", "1")))  # a longer campaign on demand
 
 
 class Guarded:
@@ -56,8 +59,8 @@ def draw_scn(g, budget=1 << 20):
             return S, C, N
 
 
-BN_CASES = [draw_scn(np.random.default_rng(100 + i)) + (int(np.random.default_rng(200 + i).integers(0, 4)),)
-            for i in range(28)]
+BN_CASES = [draw_scn(np.random.default_rng(1000 + i)) + (int(np.random.default_rng(200000 + i).integers(0, 4)),)
+            for i in range(28 * SCALE)]
 
 
 @pytest.mark.parametrize("S,C,N,offset", BN_CASES)
@@ -115,8 +118,8 @@ def test_batch_norm_family_on_drawn_shapes(oracle, S, C, N, offset):
 
 
 CAST_CASES = []
-for i in range(24):
-    _g = np.random.default_rng(300 + i)
+for i in range(24 * SCALE):
+    _g = np.random.default_rng(3000 + i)
     CAST_CASES.append((log_uniform(_g, 1, 60000), log_uniform(_g, 1, 5), log_uniform(_g, 1, 6),
                        int(_g.integers(0, 16)), int(_g.integers(0, 4))))
 
@@ -150,8 +153,8 @@ def test_casts_on_drawn_shapes(oracle, S, C, N, off_u8, off_f32):
 
 
 ROW_CASES = []
-for i in range(24):
-    _g = np.random.default_rng(400 + i)
+for i in range(24 * SCALE):
+    _g = np.random.default_rng(40000 + i)
     K = log_uniform(_g, 1, 20000)
     ROW_CASES.append((K, max(1, min(log_uniform(_g, 1, 3000), (1 << 19) // K)), int(_g.integers(0, 4))))
 
@@ -192,8 +195,8 @@ def test_row_softmax_head_on_drawn_shapes(oracle, K, R, offset):
 
 
 ND_CASES = []
-for i in range(20):
-    _g = np.random.default_rng(500 + i)
+for i in range(20 * SCALE):
+    _g = np.random.default_rng(500000 + i)
     C = log_uniform(_g, 1, 150)
     ND_CASES.append((max(1, min(log_uniform(_g, 1, 40000), (1 << 19) // C)), C, log_uniform(_g, 1, 4),
                      int(_g.integers(0, 4))))
