@@ -19,6 +19,7 @@ pytestmark = pytest.mark.gpu
 
 GUARD = 64  # elements on either side of an output
 SCALE = max(1, int(os.environ.get("ANODE_DRAWN_CASES_SCALE", "1")))  # a longer campaign on demand
+BUDGET = int(os.environ.get("ANODE_DRAWN_ELEMENTS", str(1 << 20)))      # most elements of a drawn array
 
 
 class Guarded:
@@ -49,10 +50,10 @@ def log_uniform(g, lo, hi):
     return int(round(float(np.exp(g.uniform(np.log(lo), np.log(hi + 1))))) // 1) or lo
 
 
-def draw_scn(g, budget=1 << 20):
+def draw_scn(g, budget=BUDGET):
     """(S, C, N) with S*C*N <= budget; S, C, N spread over orders of magnitude."""
     while True:
-        S = min(log_uniform(g, 1, 9000), 9000)
+        S = min(log_uniform(g, 1, 9000 * (BUDGET >> 20)), 9000 * (BUDGET >> 20))
         C = min(log_uniform(g, 1, 700), 700)
         N = min(log_uniform(g, 1, 70), 70)
         if S * C * N <= budget:
@@ -156,7 +157,7 @@ ROW_CASES = []
 for i in range(24 * SCALE):
     _g = np.random.default_rng(40000 + i)
     K = log_uniform(_g, 1, 20000)
-    ROW_CASES.append((K, max(1, min(log_uniform(_g, 1, 3000), (1 << 19) // K)), int(_g.integers(0, 4))))
+    ROW_CASES.append((K, max(1, min(log_uniform(_g, 1, 3000), (BUDGET >> 1) // K)), int(_g.integers(0, 4))))
 
 
 @pytest.mark.parametrize("K,R,offset", ROW_CASES)
@@ -198,7 +199,7 @@ ND_CASES = []
 for i in range(20 * SCALE):
     _g = np.random.default_rng(500000 + i)
     C = log_uniform(_g, 1, 150)
-    ND_CASES.append((max(1, min(log_uniform(_g, 1, 40000), (1 << 19) // C)), C, log_uniform(_g, 1, 4),
+    ND_CASES.append((max(1, min(log_uniform(_g, 1, 40000), (BUDGET >> 1) // C)), C, log_uniform(_g, 1, 4),
                      int(_g.integers(0, 4))))
 
 
