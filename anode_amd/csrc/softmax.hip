@@ -39,16 +39,49 @@ struct RowNll {
   __device__ bool on() const { return cat != nullptr; }
   __device__ uint32_t label(uint64_t r) const { return cat[r]; }
   // called by the thread that holds class k of row r, with the stored probability
-  __device__ void emit(uint64_t r, uint32_t K, uint32_t label, uint32_t k, float prob) const {
+  __device__ void emit_nll(uint64_t r, uint32_t K, uint32_t label, uint32_t k, float prob) const {
     if (k == label) {
       nll[r] = -logf(prob);
     } else if (k == 0 && label >= K) {
       nll[r] = ignore ? 0.0f : __builtin_nanf("");
     }
-    if (dx != nullptr) dx[size_t(r) * K + k] = dy[r] * (prob - float(label == k));
+  }
+  // softmax.cu:177-225: the gradient of class k for upstream gradient dyr
+  __device__ static float grad(float dyr, uint32_t label, uint32_t k, float prob) {
+    return dyr * (prob - float(label == k));
+  }
+  // the same, and the gradient stored element by element (kernels whose lanes hold consecutive classes)
+  __device__ void emit(uint64_t r, uint32_t K, uint32_t label, uint32_t k, float prob) const {
+    emit_nll(r, K, label, k, prob);
+    if (dx != nullptr) dx[size_t(r) * K + k] = grad(dy[r], label, k, prob);
   }
 };
 
+// max(a, b) as the single hardware instruction: a NaN operand yields the other operand and a signalling NaN is
+// quieted, which is fmaxf(); the library call costs two more instructions per element to canonicalise its inputs.
+__device__ inline float max1(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ inline float vmax(float a, float b) { return max1(a, b); }
+__device__ inline f32x4 vmax(f32x4 a, f32x4 b) {
+  return f32x4{max1(a.x, b.x), max1(a.y, b.y), max1(a.z, b.z), max1(a.w, b.w)};
+}
+
+// exp(d) for d <= 0 (the difference to a row's maximum): 2^(d * log2 e) with the hardware exponential, corrected
+// for the rounding of the product, r = fma(d, log2 e, -t), by the factor 1 + r ln 2.  Seven instructions instead of
+// the sixteen of expf(), which the softmax kernels feel: 76 exponentials per thread made the n-d kernel 40 % VALU-busy.
+// Relative error <= 3e-7 (+ 2e-8 |d| from the rounding of log2 e) while the result is a normal number; below
+// 2^-126 the hardware exponential returns 0, far under any probability that is compared (sums start at exp(0) = 1).
+// d = -inf gives 0 (the residual, inf - inf, is clamped before use), NaN gives NaN.
+__device__ inline float exp_nonpos(float d) {
+  constexpr float kLog2e = 1.44269502f, kLn2 = 0.693147182f;
+  const float t = d * kLog2e;
+  const float r = __builtin_amdgcn_fmed3f(fmaf(d, kLog2e, -t), -1.0f, 1.0f);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return fmaf(e, r * kLn2, e);
+}
 // K <= 64.  G = lanes per row (power of two >= K), log2g its logarithm.
 __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K, uint32_t R, uint32_t log2g,
                                                                      const float *__restrict__ x,
@@ -67,10 +100,10 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
     const size_t idx = size_t(r) * K + k;
     const float v = valid ? x[idx] : kNegInf;
     const float m = group_max(v, int(G));
-    const float z = valid ? expf(v - m) : 0.0f;
+    const float z = valid ? exp_nonpos(v - m) : 0.0f;
     const float s = group_sum(z, int(G));
     if (valid) {
-      const float pr = z / s;
+      const float pr = z * (1.0f / s);  // one correctly rounded reciprocal per row
       y[idx] = pr;
       if (nl.on()) nl.emit(r, K, nl.label(r), k, pr);
     }
@@ -127,25 +160,19 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) {
         if (uint32_t(k) < K) {
-          v[k] = expf(v[k] - m);
+          v[k] = exp_nonpos(v[k] - m);
           sum += v[k];
         }
       }
+      const float rsum = 1.0f / sum;  // one correctly rounded reciprocal per row
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) {
-        if (uint32_t(k) < K) row[k] = v[k] / sum;
+        if (uint32_t(k) < K) row[k] = v[k] * rsum;
       }
       if (nl.on()) {
         const uint64_t r = r0 + threadIdx.x;
         const uint32_t label = nl.label(r);
-        if (nl.dx != nullptr) {
-#pragma unroll
-          for (int k = 0; k < KMAX; ++k) {
-            if (uint32_t(k) < K) nl.emit(r, K, label, uint32_t(k), row[k]);
-          }
-        } else {
-          nl.emit(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
-        }
+        nl.emit_nll(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
       }
     }
     __syncthreads();
@@ -169,6 +196,41 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
       yt[e] = tile[q * pitch + c];
     }
     __syncthreads();  // the tile is overwritten by the next pass
+    if (nl.on() && nl.dx != nullptr) {
+      // the gradient takes the same way out: each thread turns its row into dy * (p - onehot) in place
+      if (threadIdx.x < rows) {
+        float *row = tile + threadIdx.x * pitch;
+        const uint64_t r = r0 + threadIdx.x;
+        const uint32_t label = nl.label(r);
+        const float dyr = nl.dy[r];
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) {
+          if (uint32_t(k) < K) row[k] = RowNll::grad(dyr, label, uint32_t(k), row[k]);
+        }
+      }
+      __syncthreads();
+      float *dt = nl.dx + r0 * K;
+      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
+        uint32_t q, c;
+        div_k.divmod(g * 4u, q, c);
+        f32x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[j] = tile[q * pitch + c];
+          if (++c == K) {
+            c = 0;
+            ++q;
+          }
+        }
+        store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, v);
+      }
+      for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
+        uint32_t q, c;
+        div_k.divmod(e, q, c);
+        dt[e] = tile[q * pitch + c];
+      }
+      __syncthreads();
+    }
   }
 }
 
@@ -186,6 +248,9 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
   for (uint64_t r = wave; r < R; r += n_waves) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
+    // the row's label and upstream gradient are requested together with the row, not after the reductions
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
     float v[VPL];
     float m = kNegInf;
 #pragma unroll
@@ -209,24 +274,31 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
       const uint32_t k = (lane + uint32_t(i / W) * kWave) * uint32_t(W) + uint32_t(i % W);
-      v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
+      v[i] = (k < K) ? exp_nonpos(v[i] - m) : 0.0f;
       s += v[i];
     }
     s = wave_sum(s);
-    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
       if (k < K) {
 #pragma unroll
         for (int j = 0; j < W; ++j) {
-          v[i * W + j] = v[i * W + j] / s;
-          if (nl.on()) nl.emit(r, K, label, k + uint32_t(j), v[i * W + j]);
+          v[i * W + j] = v[i * W + j] * rs;
+          if (nl.on()) nl.emit_nll(r, K, label, k + uint32_t(j), v[i * W + j]);
         }
         if (VEC) {
           store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
+          if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
+            store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
+                             f32x4{RowNll::grad(dyr, label, k, v[i * W]), RowNll::grad(dyr, label, k + 1u, v[i * W + 1]),
+                                   RowNll::grad(dyr, label, k + 2u, v[i * W + 2]),
+                                   RowNll::grad(dyr, label, k + 3u, v[i * W + 3])});
+          }
         } else {
           yr[k] = v[i];
+          if (nl.on() && nl.dx != nullptr) nl.dx[size_t(r) * K + k] = RowNll::grad(dyr, label, k, v[i]);
         }
       }
     }
@@ -237,8 +309,8 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
 // (-inf, 0) and must not produce exp(-inf - -inf).
 __device__ inline void online_merge(float &m, float &s, float m2, float s2) {
   const float mm = fmaxf(m, m2);
-  const float a = (m == mm) ? s : s * expf(m - mm);
-  const float b = (m2 == mm) ? s2 : s2 * expf(m2 - mm);
+  const float a = (m == mm) ? s : s * exp_nonpos(m - mm);
+  const float b = (m2 == mm) ? s2 : s2 * exp_nonpos(m2 - mm);
   s = ((s == 0.0f) ? 0.0f : a) + ((s2 == 0.0f) ? 0.0f : b);
   m = mm;
 }
@@ -255,6 +327,9 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
+    // the row's label and upstream gradient are requested together with the row, not after the reductions
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
     float v[VPT];
     float m = kNegInf;
 #pragma unroll
@@ -278,24 +353,31 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
       const uint32_t k = (threadIdx.x + uint32_t(i / W) * kBlock) * uint32_t(W) + uint32_t(i % W);
-      v[i] = (k < K) ? expf(v[i] - m) : 0.0f;
+      v[i] = (k < K) ? exp_nonpos(v[i] - m) : 0.0f;
       s += v[i];
     }
     s = block_sum(s, lds);
-    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
       const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
       if (k < K) {
 #pragma unroll
         for (int j = 0; j < W; ++j) {
-          v[i * W + j] = v[i * W + j] / s;
-          if (nl.on()) nl.emit(r, K, label, k + uint32_t(j), v[i * W + j]);
+          v[i * W + j] = v[i * W + j] * rs;
+          if (nl.on()) nl.emit_nll(r, K, label, k + uint32_t(j), v[i * W + j]);
         }
         if (VEC) {
           store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
+          if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
+            store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
+                             f32x4{RowNll::grad(dyr, label, k, v[i * W]), RowNll::grad(dyr, label, k + 1u, v[i * W + 1]),
+                                   RowNll::grad(dyr, label, k + 2u, v[i * W + 2]),
+                                   RowNll::grad(dyr, label, k + 3u, v[i * W + 3])});
+          }
         } else {
           yr[k] = v[i];
+          if (nl.on() && nl.dx != nullptr) nl.dx[size_t(r) * K + k] = RowNll::grad(dyr, label, k, v[i]);
         }
       }
     }
@@ -314,11 +396,11 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
     for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
       const float v = xr[k];
       if (v > m) {
-        s = (s == 0.0f) ? 1.0f : fmaf(s, expf(m - v), 1.0f);
+        s = (s == 0.0f) ? 1.0f : fmaf(s, exp_nonpos(m - v), 1.0f);
         m = v;
       } else if (!(v == kNegInf && m == kNegInf)) {
         // a -inf seen before any larger value adds exp(-inf - max) = 0
-        s += expf(v - m);
+        s += exp_nonpos(v - m);
       }
     }
 #pragma unroll
@@ -337,9 +419,10 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
 #pragma unroll
     for (int w = 1; w < kBlock / kWave; ++w) online_merge(m, s, lds_m[w], lds_s[w]);
     __syncthreads();
+    const float rs = 1.0f / s;
     const uint32_t label = nl.on() ? nl.label(r) : 0u;
     for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
-      const float pr = expf(xr[k] - m) / s;
+      const float pr = exp_nonpos(xr[k] - m) * rs;
       yr[k] = pr;
       if (nl.on()) nl.emit(r, K, label, k, pr);
     }
@@ -361,7 +444,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     if (blocks > max_blocks) blocks = max_blocks;
     const size_t lds_bytes = size_t(kBlock) * (K | 1u) * sizeof(float);
     const FastDiv div_k(K);
-    const int vec = (aligned16(x) && aligned16(y)) ? 1 : 0;
+    const int vec = (aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx))) ? 1 : 0;
     with_stream_policy(nt & kNtStore, [&](auto policy) {
       constexpr int NT = decltype(policy)::value;
       if (K <= 4) {
@@ -384,7 +467,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   } else if (K <= 2048) {
     uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > max_blocks) blocks = max_blocks;
-    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
+    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx));
 #define ANODE_ROW_WAVE(VPL)                                                              \
   do {                                                                                   \
     if (vec) {                                                                           \
@@ -407,7 +490,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
 #undef ANODE_ROW_WAVE
   } else {
     const uint32_t blocks = R < max_blocks ? R : max_blocks;
-    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y);
+    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx));
 #define ANODE_ROW_BLOCKREG(VPT)                                                          \
   do {                                                                                   \
     if (vec) {                                                                           \
@@ -485,31 +568,6 @@ template <> struct PixVec<f32x4> {
 __device__ inline uint32_t lane_get_u(uint32_t v, int) { return v; }
 __device__ inline uint32_t lane_get_u(u32x4 v, int k) { return v[k]; }
 
-// max(a, b) as the single hardware instruction: a NaN operand yields the other operand and a signalling NaN is
-// quieted, which is fmaxf(); the library call costs two more instructions per element to canonicalise its inputs.
-__device__ inline float max1(float a, float b) {
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-__device__ inline float vmax(float a, float b) { return max1(a, b); }
-__device__ inline f32x4 vmax(f32x4 a, f32x4 b) {
-  return f32x4{max1(a.x, b.x), max1(a.y, b.y), max1(a.z, b.z), max1(a.w, b.w)};
-}
-
-// exp(d) for d <= 0 (the difference to a row's maximum): 2^(d * log2 e) with the hardware exponential, corrected
-// for the rounding of the product, r = fma(d, log2 e, -t), by the factor 1 + r ln 2.  Seven instructions instead of
-// the sixteen of expf(), which the n-d kernels feel: 76 exponentials per thread made them 40 % VALU-busy.
-// Relative error <= 3e-7 (+ 2e-8 |d| from the rounding of log2 e) while the result is a normal number; below
-// 2^-126 the hardware exponential returns 0, far under any probability that is compared (sums start at exp(0) = 1).
-// d = -inf gives 0 (the residual, inf - inf, is clamped before use), NaN gives NaN.
-__device__ inline float exp_nonpos(float d) {
-  constexpr float kLog2e = 1.44269502f, kLn2 = 0.693147182f;
-  const float t = d * kLog2e;
-  const float r = __builtin_amdgcn_fmed3f(fmaf(d, kLog2e, -t), -1.0f, 1.0f);
-  const float e = __builtin_amdgcn_exp2f(t);
-  return fmaf(e, r * kLn2, e);
-}
 __device__ inline float vexp(float a) { return exp_nonpos(a); }
 __device__ inline f32x4 vexp(f32x4 a) { return f32x4{exp_nonpos(a.x), exp_nonpos(a.y), exp_nonpos(a.z), exp_nonpos(a.w)}; }
 __device__ inline float vrcp(float a) { return 1.0f / a; }
