@@ -242,12 +242,24 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
                                                                   float *__restrict__ y, RowNll nl) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int NG = VPL / W;  // groups per lane
+  static_assert((NG & (NG - 1)) == 0, "the wrapped lane assignment needs a power-of-two number of groups per lane");
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
   const uint32_t n_waves = gridDim.x * (kBlock / kWave);
   for (uint64_t r = wave; r < R; r += n_waves) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
+    // VEC: step i of the wave covers one aligned run of 16-byte groups of the ARRAY, not of the row: the groups are
+    // taken `a` places earlier, a = the row's distance from the 128-byte line before it (in groups, for an array
+    // that starts on a line), and the first a lanes wrap round to the row's tail.  A row of 1000 floats starts 32
+    // bytes into a line three times out of four, and half-written 64-byte pieces cost a tenth of the bandwidth
+    // ([65536, 1000]: 5.5 TB/s, against 6.1 for 992 or 1024 columns).  The shift depends on the row number
+    // only, so results do not depend on where the arrays lie.
+    const uint32_t a = VEC ? (uint32_t(r) * (K / 4u)) & 7u : 0u;
+    auto kof = [&](int i) -> uint32_t {
+      const uint32_t slot = lane + uint32_t(i) * kWave;
+      return VEC ? ((slot + uint32_t(NG) * kWave - a) & (uint32_t(NG) * kWave - 1u)) * 4u : slot;
+    };
     // the row's label and upstream gradient are requested together with the row, not after the reductions
     const uint32_t label = nl.on() ? nl.label(r) : 0u;
     const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
@@ -255,7 +267,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
     float m = kNegInf;
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-      const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
+      const uint32_t k = kof(i);
       if (VEC) {
         const f32x4 t = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k))
                                 : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
@@ -273,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
-      const uint32_t k = (lane + uint32_t(i / W) * kWave) * uint32_t(W) + uint32_t(i % W);
+      const uint32_t k = kof(i / W) + uint32_t(i % W);
       v[i] = (k < K) ? exp_nonpos(v[i] - m) : 0.0f;
       s += v[i];
     }
@@ -281,7 +293,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
     const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-      const uint32_t k = (lane + uint32_t(i) * kWave) * uint32_t(W);
+      const uint32_t k = kof(i);
       if (k < K) {
 #pragma unroll
         for (int j = 0; j < W; ++j) {
@@ -323,10 +335,22 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
                                                                       float *__restrict__ y, RowNll nl) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int NG = VPT / W;
+  static_assert((NG & (NG - 1)) == 0, "the wrapped lane assignment needs a power-of-two number of groups per thread");
   __shared__ float lds[kBlock / kWave];
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
+    // VEC: step i of the workgroup covers one aligned run of 16-byte groups of the ARRAY, not of the row: the groups are
+    // taken `a` places earlier, a = the row's distance from the 128-byte line before it (in groups, for an array
+    // that starts on a line), and the first a lanes wrap round to the row's tail.  A row of 1000 floats starts 32
+    // bytes into a line three times out of four, and half-written 64-byte pieces cost a tenth of the bandwidth
+    // ([65536, 1000]: 5.5 TB/s, against 6.1 for 992 or 1024 columns).  The shift depends on the row number
+    // only, so results do not depend on where the arrays lie.
+    const uint32_t a = VEC ? (uint32_t(r) * (K / 4u)) & 7u : 0u;
+    auto kof = [&](int i) -> uint32_t {
+      const uint32_t slot = threadIdx.x + uint32_t(i) * kBlock;
+      return VEC ? ((slot + uint32_t(NG) * kBlock - a) & (uint32_t(NG) * kBlock - 1u)) * 4u : slot;
+    };
     // the row's label and upstream gradient are requested together with the row, not after the reductions
     const uint32_t label = nl.on() ? nl.label(r) : 0u;
     const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
@@ -334,7 +358,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
     float m = kNegInf;
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-      const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
+      const uint32_t k = kof(i);
       if (VEC) {
         const f32x4 t = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k))
                                 : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
@@ -352,7 +376,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const uint32_t k = (threadIdx.x + uint32_t(i / W) * kBlock) * uint32_t(W) + uint32_t(i % W);
+      const uint32_t k = kof(i / W) + uint32_t(i % W);
       v[i] = (k < K) ? exp_nonpos(v[i] - m) : 0.0f;
       s += v[i];
     }
@@ -360,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
     const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-      const uint32_t k = (threadIdx.x + uint32_t(i) * kBlock) * uint32_t(W);
+      const uint32_t k = kof(i);
       if (k < K) {
 #pragma unroll
         for (int j = 0; j < W; ++j) {
