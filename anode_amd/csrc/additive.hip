@@ -396,7 +396,7 @@ __global__ __launch_bounds__(kBlock) void online_average_kernel(uint32_t len, fl
 // First index of the strict maximum of each row of a [K (fastest), R] array;
 // NaN never wins; a row without any value above -inf gives 0.  One wave per row.
 // VEC: rows start on 16-byte boundaries (K a multiple of 4, x aligned), so a lane reads four consecutive classes.
-template <bool VEC>
+template <bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void arg_max_rows_kernel(uint32_t K, uint32_t R, const float *__restrict__ x,
                                                               uint32_t *__restrict__ out) {
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -407,16 +407,28 @@ __global__ __launch_bounds__(kBlock) void arg_max_rows_kernel(uint32_t K, uint32
     float top = -__builtin_huge_valf();
     uint32_t idx = 0xffffffffu;  // nothing above -inf seen yet
     if (VEC) {
+      constexpr int U = 4;  // loads in flight per lane
       const f32x4 *xr4 = reinterpret_cast<const f32x4 *>(xr);
-      const uint32_t n4 = K / 4u;
-#pragma unroll 4
-      for (uint32_t g = lane; g < n4; g += kWave) {
-        const f32x4 v = xr4[g];
+      const int32_t n4 = int32_t(K / 4u);
+      // each step of the wave reads one 128-byte-aligned run of the array (for an array that starts on a line):
+      // the groups are taken `a` places earlier than the row starts, and the first a lanes sit out the first step
+      const int32_t a = int32_t((uint32_t(r) * (K / 4u)) & 7u);
+      for (int32_t g0 = int32_t(lane) - a; g0 < n4; g0 += U * kWave) {
+        f32x4 v[U];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {  // ascending class index inside the lane: the first maximum is kept
-          if (v[j] > top) {
-            top = v[j];
-            idx = g * 4u + uint32_t(j);
+        for (int u = 0; u < U; ++u) {
+          const int32_t g = g0 + u * kWave;
+          // a slot outside the row holds -inf, which never wins
+          v[u] = (g >= 0 && g < n4) ? load_stream<NT>(&xr4[g]) : f32x4{-__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf()};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {  // ascending class index inside the lane: the first maximum is kept
+            if (v[u][j] > top) {
+              top = v[u][j];
+              idx = uint32_t(g0 + u * kWave) * 4u + uint32_t(j);
+            }
           }
         }
       }
@@ -724,9 +736,14 @@ ANODE_EXPORT void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, con
   const uint32_t cap = 1u << 24;  // one row per wave; the kernel loops only beyond that
   if (blocks > cap) blocks = cap;
   if (dim0 % 4u == 0 && aligned16(x)) {
-    arg_max_rows_kernel<true><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
+    const int nt = stream_policy(size_t(dim0) * dim1 * sizeof(float), tuning().reduce_nontemporal) & kNtLoad;
+    if (nt) {
+      arg_max_rows_kernel<true, kNtLoad><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
+    } else {
+      arg_max_rows_kernel<true, 0><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
+    }
   } else {
-    arg_max_rows_kernel<false><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
+    arg_max_rows_kernel<false, 0><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);
   }
   note_launch(__func__);
 }
