@@ -97,6 +97,89 @@ def test_softmax_nd_beyond_2_31(big):
     del p, sums
 
 
+def test_short_channels_beyond_2_31(big):
+    # 7x7 maps: the reductions run as lane tiles (one launch, all samples per workgroup), the maps walk channels of
+    # 49 elements; sample offsets n * C * S pass 2^31
+    S, C, N = 49, 2048, 21409            # 2 148 435 968 elements
+    n = S * C * N
+    assert (1 << 31) < n <= N_BIG
+    x = big[:n]
+    mean, var = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, x, mean)
+    call("anode_gpu_batch_var_3d1_packed_f32", S, C, N, 1e-5, x, mean, var)
+    m1, v1 = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    call("anode_gpu_batch_mean_var_3d1_packed_f32", S, C, N, 1e-5, x, m1, v1)
+    y = torch.empty(n, device="cuda")
+    call("anode_gpu_batch_norm_3d1_packed_f32", S, C, N, x, mean, var, y)
+    torch.cuda.synchronize()
+    xv, yv = x.view(N, C, S), y.view(N, C, S)
+    for c in (0, 1, 1023, 2046, 2047):
+        col = xv[:, c, :].double()
+        m = col.mean().item()
+        v = ((col - float(mean[c])) ** 2).mean().item() + 1e-5
+        assert abs(float(mean[c]) - m) <= 1e-5 * abs(m) + 1e-7
+        assert abs(float(var[c]) - v) <= 1e-5 * v
+        assert abs(float(m1[c]) - m) <= 1e-5 * abs(m) + 1e-7 and abs(float(v1[c]) - v) <= 1e-5 * v
+        want = (xv[:, c, :] - mean[c]) / torch.sqrt(var[c])      # the map's own fp32 formula
+        assert bool(((yv[:, c, :] - want).abs() <= 2e-6 * want.abs() + 1e-7).all())
+        del col, want
+    # the last sample (the far end of the array) on its own, every channel
+    want = (xv[N - 1] - mean.view(C, 1)) / torch.sqrt(var.view(C, 1))
+    assert bool(((yv[N - 1] - want).abs() <= 2e-6 * want.abs() + 1e-7).all())
+    del y
+
+
+def test_row_softmax_head_beyond_2_31(big):
+    K, R = 1000, 2148000                 # 2 148 000 000 elements; rows in registers, one wave per row
+    n = K * R
+    assert (1 << 31) < n <= N_BIG
+    x = big[:n]
+    lab = torch.randint(0, K, (R,), device="cuda", dtype=torch.int32)
+    dy = torch.full((R,), 0.5, device="cuda")
+    p, nll, dx = torch.empty(n, device="cuda"), torch.empty(R, device="cuda"), torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32", K, R, x, lab, dy, p, nll, dx)
+    idx = torch.empty(R, device="cuda", dtype=torch.int32)
+    call("anode_gpu_arg_max_packed_u32", K, R, x, idx)
+    torch.cuda.synchronize()
+    pv, xv, dv = p.view(R, K), x.view(R, K), dx.view(R, K)
+    for lo in (0, (1 << 31) // K - 500, R - 1000):     # the first rows, rows across 2^31, the last rows
+        rows = slice(lo, lo + 1000)
+        ref = torch.softmax(xv[rows].double(), dim=1)
+        assert bool(((pv[rows].double() - ref).abs() <= 1e-5 * ref).all())
+        picked = torch.gather(pv[rows], 1, lab[rows].long().unsqueeze(1)).squeeze(1)
+        assert torch.allclose(nll[rows], -torch.log(picked), rtol=1e-5, atol=1e-6)
+        onehot = torch.nn.functional.one_hot(lab[rows].long(), K).float()
+        assert torch.equal(dv[rows], 0.5 * (pv[rows] - onehot))
+        top = torch.gather(xv[rows], 1, idx[rows].long().unsqueeze(1)).squeeze(1)
+        assert torch.equal(top, xv[rows].max(dim=1).values)
+    sums = pv.sum(dim=1)
+    assert bool(((sums - 1).abs() < 1e-5).all())
+    del p, dx, sums
+
+
+def test_casts_beyond_2_31(big):
+    # quantize(dequantize(q)) == q for every code, and upcast is exact: 2^31 + 2^20 + 7 bytes in, 16-byte and tail paths
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    q = torch.randint(0, 256, (N_BIG,), device="cuda", dtype=torch.uint8, generator=g)
+    f = torch.empty(N_BIG, device="cuda")
+    call("anode_gpu_dequantize_u8_packed_f32", N_BIG, -1.0, 3.0, q, f)
+    back = torch.empty(N_BIG, device="cuda", dtype=torch.uint8)
+    call("anode_gpu_quantize_u8_packed_f32", N_BIG, -1.0, 3.0, f, back)
+    torch.cuda.synchronize()
+    assert torch.equal(back, q)
+    assert float(f.min()) == -1.0 and abs(float(f.max()) - 3.0) <= 3e-7   # code 255: fma(255, fl(4/255), -1), one rounding
+    del back
+    u = f.view(torch.int32)              # reuse the 8.6 GB buffer
+    call("anode_gpu_upcast_u8_packed_u32", N_BIG, q, u)
+    torch.cuda.synchronize()
+    step = 1 << 28
+    for lo in range(0, N_BIG, step):
+        hi = min(N_BIG, lo + step)
+        assert torch.equal(u[lo:hi], q[lo:hi].to(torch.int32))
+    del q, f, u
+
+
 # ---- close to the largest array the 32-bit counts of the ABI can describe: 2^32 - 3 elements (17 GB) ----
 
 N_MAX = (1 << 32) - 3
