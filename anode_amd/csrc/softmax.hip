@@ -111,49 +111,44 @@ __global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K,
 }
 
 // K <= KMAX <= 32: one thread per row.  A workgroup takes 256 consecutive rows, which are 256*K contiguous floats:
-// they are copied to LDS with full-width coalesced loads (row pitch K|1, so that threads reading their own row hit
-// distinct banks), each thread normalises its row in registers, and the tile goes back the same way.  No cross-lane
-// traffic at all, which is what bounds the lane-group kernel below for short rows.
+// they are copied to LDS as they lie in memory, 16 bytes per lane, each thread normalises its row in registers, and
+// the tile goes back the same way.  No cross-lane traffic at all, which is what bounds the lane-group kernel below
+// for short rows.  A thread walks its row from element (row number mod K) on, wrapping round: with every thread
+// starting at element 0 the lanes of a wave would meet in the same LDS banks whenever K is even (all 32 in one bank
+// for K = 32).  The sum of a row is therefore taken in an order that depends on the row number, and on nothing else.
 template <int KMAX, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, FastDiv div_k, int vec,
                                                                  const float *__restrict__ x,
                                                                  float *__restrict__ y, RowNll nl) {
-  extern __shared__ float tile[];  // kBlock * (K|1) floats
-  const uint32_t pitch = K | 1u;
+  extern __shared__ __align__(16) float tile[];  // kBlock * K floats
+  f32x4 *tile4 = reinterpret_cast<f32x4 *>(tile);
   for (uint64_t r0 = uint64_t(blockIdx.x) * kBlock; r0 < R; r0 += uint64_t(gridDim.x) * kBlock) {
     const uint32_t rows = (R - r0 < uint64_t(kBlock)) ? uint32_t(R - r0) : uint32_t(kBlock);
     const uint32_t n = rows * K;
     const float *xt = x + r0 * K;
     float *yt = y + r0 * K;
     const uint32_t n4 = vec ? n / 4u : 0u;  // the tile starts 1024*K bytes into an aligned array: 16-byte aligned
-    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
-      const f32x4 v = reinterpret_cast<const f32x4 *>(xt)[g];
-      uint32_t q, c;
-      div_k.divmod(g * 4u, q, c);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        tile[q * pitch + c] = v[j];
-        if (++c == K) {
-          c = 0;
-          ++q;
-        }
-      }
-    }
-    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
-      uint32_t q, c;
-      div_k.divmod(e, q, c);
-      tile[q * pitch + c] = xt[e];
-    }
+    // the row's label and upstream gradient are requested together with the tile
+    const uint64_t r = r0 + threadIdx.x;
+    const bool mine = threadIdx.x < rows;
+    const uint32_t label = (mine && nl.on()) ? nl.label(r) : 0u;
+    const float dyr = (mine && nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
+    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) tile4[g] = reinterpret_cast<const f32x4 *>(xt)[g];
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) tile[e] = xt[e];
     __syncthreads();
-    if (threadIdx.x < rows) {
-      float *row = tile + threadIdx.x * pitch;
-      float v[KMAX];
+    float *row = tile + threadIdx.x * K;
+    uint32_t q0, first;
+    div_k.divmod(uint32_t(r), q0, first);  // first = row number mod K (r < 2^32: K * R fits 32 bits)
+    float v[KMAX];
+    if (mine) {
       float m = kNegInf;
+      uint32_t at = first;
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) {
         if (uint32_t(k) < K) {
-          v[k] = row[k];
+          v[k] = row[at];
           m = fmaxf(m, v[k]);
+          at = (at + 1u == K) ? 0u : at + 1u;
         }
       }
       float sum = 0.0f;
@@ -165,70 +160,37 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
         }
       }
       const float rsum = 1.0f / sum;  // one correctly rounded reciprocal per row
+      at = first;
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) {
-        if (uint32_t(k) < K) row[k] = v[k] * rsum;
-      }
-      if (nl.on()) {
-        const uint64_t r = r0 + threadIdx.x;
-        const uint32_t label = nl.label(r);
-        nl.emit_nll(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
-      }
-    }
-    __syncthreads();
-    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
-      uint32_t q, c;
-      div_k.divmod(g * 4u, q, c);
-      f32x4 v;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[j] = tile[q * pitch + c];
-        if (++c == K) {
-          c = 0;
-          ++q;
+        if (uint32_t(k) < K) {
+          v[k] = v[k] * rsum;
+          row[at] = v[k];
+          at = (at + 1u == K) ? 0u : at + 1u;
         }
       }
-      store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, v);
+      if (nl.on()) nl.emit_nll(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
     }
-    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
-      uint32_t q, c;
-      div_k.divmod(e, q, c);
-      yt[e] = tile[q * pitch + c];
-    }
-    __syncthreads();  // the tile is overwritten by the next pass
+    __syncthreads();
+    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, tile4[g]);
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) yt[e] = tile[e];
+    __syncthreads();  // the tile is overwritten below, or by the next pass
     if (nl.on() && nl.dx != nullptr) {
       // the gradient takes the same way out: each thread turns its row into dy * (p - onehot) in place
-      if (threadIdx.x < rows) {
-        float *row = tile + threadIdx.x * pitch;
-        const uint64_t r = r0 + threadIdx.x;
-        const uint32_t label = nl.label(r);
-        const float dyr = nl.dy[r];
+      if (mine) {
+        uint32_t at = first;
 #pragma unroll
         for (int k = 0; k < KMAX; ++k) {
-          if (uint32_t(k) < K) row[k] = RowNll::grad(dyr, label, uint32_t(k), row[k]);
+          if (uint32_t(k) < K) {
+            row[at] = RowNll::grad(dyr, label, at, v[k]);
+            at = (at + 1u == K) ? 0u : at + 1u;
+          }
         }
       }
       __syncthreads();
       float *dt = nl.dx + r0 * K;
-      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) {
-        uint32_t q, c;
-        div_k.divmod(g * 4u, q, c);
-        f32x4 v;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v[j] = tile[q * pitch + c];
-          if (++c == K) {
-            c = 0;
-            ++q;
-          }
-        }
-        store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, v);
-      }
-      for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) {
-        uint32_t q, c;
-        div_k.divmod(e, q, c);
-        dt[e] = tile[q * pitch + c];
-      }
+      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, tile4[g]);
+      for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) dt[e] = tile[e];
       __syncthreads();
     }
   }
@@ -466,7 +428,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   if (K <= 32) {
     uint32_t blocks = (R + kBlock - 1) / kBlock;
     if (blocks > max_blocks) blocks = max_blocks;
-    const size_t lds_bytes = size_t(kBlock) * (K | 1u) * sizeof(float);
+    const size_t lds_bytes = size_t(kBlock) * K * sizeof(float);
     const FastDiv div_k(K);
     const int vec = (aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx))) ? 1 : 0;
     with_stream_policy(nt & kNtStore, [&](auto policy) {
