@@ -589,11 +589,16 @@ __device__ inline f32x4 pair_swap(f32x4 v) {
 // are added last; the normalisation multiplies by one correctly rounded reciprocal per pixel.  With NLL the label
 // gather is fused: nll = -log(the stored probability of the label), NaN when the label is out of range, exactly
 // what the separate gather returns.
-template <int CMAX, typename V, bool NLL, int NT, int SPLIT>
+// With BWD the gradient of the summed loss for a dy known up front is written in the same pass:
+// dx = dy * (p - onehot), the arithmetic (and, with pg.ignore, the masking) of softmax_nd_cat_nll_bwd_kernel.
+template <int CMAX, typename V, bool NLL, int NT, int SPLIT, bool BWD = false>
 __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 const uint32_t *__restrict__ cat,
-                                                                float *__restrict__ nll) {
+                                                                float *__restrict__ nll,
+                                                                const float *__restrict__ dy = nullptr,
+                                                                float *__restrict__ dx = nullptr) {
+  static_assert(!BWD || NLL, "the backward pass needs the labels");
   constexpr int W = PixVec<V>::W;
   constexpr int H = (CMAX + SPLIT - 1) / SPLIT;  // classes a lane holds
   typedef typename PixVec<V>::U U;
@@ -614,6 +619,16 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     U lab;
     if (NLL) lab = *reinterpret_cast<const U *>(cat + pix);
+    V d;
+    if (BWD) {
+      d = *reinterpret_cast<const V *>(dy + pix);
+      if (pg.ignore) {
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          if (lane_get_u(lab, w) >= pg.C) lane_set<V>(d, w, 0.0f);
+        }
+      }
+    }
     V m = PixVec<V>::splat(kNegInf);
 #pragma unroll
     for (int i = 0; i < H; ++i) {
@@ -633,7 +648,18 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
 #pragma unroll
     for (int i = 0; i < H; ++i) {
       const uint32_t k = uint32_t(i) * SPLIT + h;
-      if (k < pg.C) store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), v[i] * inv);
+      if (k < pg.C) {
+        const V pr = v[i] * inv;
+        store_stream<NT>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), pr);
+        if (BWD) {
+          V gr;
+#pragma unroll
+          for (int w = 0; w < W; ++w) {
+            lane_set<V>(gr, w, lane_get<V>(d, w) * (lane_get<V>(pr, w) - float(lane_get_u(lab, w) == k)));
+          }
+          store_stream<NT>(reinterpret_cast<V *>(dx + base + size_t(pg.P) * k), gr);
+        }
+      }
     }
     if (NLL) {
       // The label's exponential is picked out of the registers of the lane that holds it (a compare and a select
@@ -778,40 +804,41 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore
 uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
 // C <= 32 only.  The 16-byte form runs two lanes per pixel group.
-template <typename V, bool NLL, int NT>
+template <typename V, bool NLL, int NT, bool BWD = false>
 void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
-                              float *nll, hipStream_t s) {
+                              float *nll, hipStream_t s, const float *dy = nullptr, float *dx = nullptr,
+                              bool ignore = false) {
   constexpr int SPLIT = PixVec<V>::W == 4 ? 2 : 1;
-  PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
+  PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W, ignore);
   pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
   const uint32_t blocks = stream_grid(uint64_t(pg.total_groups) * SPLIT, 1);
   if (C <= 4) {
-    softmax_nd_reg_kernel<4, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<4, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   } else if (C <= 8) {
-    softmax_nd_reg_kernel<8, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<8, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   } else if (C <= 16) {
-    softmax_nd_reg_kernel<16, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<16, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   } else if (C <= 20) {  // 19 / 20 classes are common label sets
-    softmax_nd_reg_kernel<20, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<20, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   } else if (C <= 24) {
-    softmax_nd_reg_kernel<24, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<24, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   } else {
-    softmax_nd_reg_kernel<32, V, NLL, NT, SPLIT><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll);
+    softmax_nd_reg_kernel<32, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
   }
 }
 
-template <typename V, bool NLL>
+template <typename V, bool NLL, bool BWD = false>
 void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
-                           float *nll, hipStream_t s) {
+                           float *nll, hipStream_t s, const float *dy = nullptr, float *dx = nullptr) {
   // the input is streamed; the probabilities are read again by the NLL gather and the backward pass, so they
   // keep the default policy unless they are far larger than the last-level cache
   const size_t bytes = size_t(P) * C * N * sizeof(float);
   if (PixVec<V>::W == 4) {
     with_stream_policy(stream_policy(bytes, tuning().nontemporal), [&](auto policy) {
-      launch_softmax_nd_reg_nt<V, NLL, decltype(policy)::value>(P, C, N, x, y, cat, nll, s);
+      launch_softmax_nd_reg_nt<V, NLL, decltype(policy)::value, BWD>(P, C, N, x, y, cat, nll, s, dy, dx);
     });
   } else {
-    launch_softmax_nd_reg_nt<V, NLL, 0>(P, C, N, x, y, cat, nll, s);
+    launch_softmax_nd_reg_nt<V, NLL, 0, BWD>(P, C, N, x, y, cat, nll, s, dy, dx);
   }
 }
 
@@ -1014,6 +1041,36 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     // shapes outside the register-resident kernel: the two passes, back to back
     anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
     anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
+  }
+}
+
+// Additive: the same and the backward pass for a dy that is known before the forward pass (ones for a summed loss,
+// 1/count for a mean), one launch instead of three.  softmax, nll and dx are bit-identical to softmax_nd,
+// softmax_nd_cat_nll and softmax_nd_cat_nll_bwd.
+ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t prefix_dim, uint32_t dim0,
+                                                                        uint32_t dim1, const float *x,
+                                                                        const uint32_t *cat_data, const float *dy,
+                                                                        float *softmax, float *nll, float *dx,
+                                                                        const KernelConfig *cfg, CUstream_st *stream) {
+  const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
+  if (len == 0) return;
+  if (prefix_dim == 1) {  // the class axis is contiguous: the row form
+    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
+  } else if (dim0 <= 32) {
+    hipStream_t s = as_stream(stream);
+    const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
+                     aligned16(nll) && aligned16(dy) && aligned16(dx);
+    if (vec) {
+      launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
+    } else {
+      launch_softmax_nd_reg<float, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
+    }
+    note_launch(__func__);
+  } else {
+    // shapes outside the register-resident kernel: the three passes, back to back
+    anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
+    anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
+    anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, cfg, stream);
   }
 }
 

@@ -282,6 +282,10 @@ def build_workload(torch, only, copy_calibration=False):
         p2, nll2 = empty(n), empty(P * N)
         fused.append(Launch("fused_softmax_fwd_cfg3b", "anode_gpu_softmax_nd_cat_nll_fused_packed_f32",
                             (P, C, N, x, lab, p2, nll2), 8 * n + 8 * P * N, n))
+        # forward and backward in one launch for the dy of a summed loss: x, labels, dy in; p, nll, dx out
+        dx2 = empty(n)
+        fused.append(Launch("fused_softmax_fwd_bwd_cfg3b", "anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32",
+                            (P, C, N, x, lab, dy, p2, nll2, dx2), 12 * n + 12 * P * N, n))
     return launches, fused
 
 
@@ -434,6 +438,8 @@ def all_symbols(torch, gpu):
     add("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", ss, (P, Cc, Nn, dy, x, lab, y), 8 * ns + 8 * P * Nn)
     add("anode_gpu_softmax_nd_cat_nll_bwd_packed_accumulate_f32", ss, (P, Cc, Nn, dy, x, lab, dx), 12 * ns + 8 * P * Nn)
     add("anode_gpu_softmax_nd_cat_nll_fused_packed_f32", ss, (P, Cc, Nn, x, lab, y, E(P * Nn)), 8 * ns + 8 * P * Nn)
+    add("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", ss, (P, Cc, Nn, x, lab, dy, y, E(P * Nn), dx),
+        12 * ns + 12 * P * Nn)
     add("anode_gpu_discrete_one_hot_3d1_packed_f32", ss, (P, Cc, Nn, lab, y), 4 * P * Nn + 4 * ns)
     t01 = (torch.rand(ns, device="cuda", generator=g) < 0.3).float()
     add("anode_gpu_smooth_negative_f1_loss_3d1_packed_f32", ss, (P, Cc, Nn, 1e-3, x, t01, E(Cc * Nn)), 8 * ns)
@@ -834,6 +840,7 @@ def main():
             "fused_bn_fwd_cfg4": ["bn_fwd_cfg4", "relu_cfg4:positive_clip_flat_map_f32"],
             "fused_bn_bwd_cfg4": ["bn_bwd_cfg4", "relu_cfg4:positive_clip_flat_map_bwd_f32"],
             "fused_softmax_fwd_cfg3b": ["softmax_cfg3b:softmax_nd_packed_f32", "softmax_cfg3b:softmax_nd_cat_nll_packed_f32"],
+            "fused_softmax_fwd_bwd_cfg3b": ["softmax_cfg3b"],
             "fused_softmax_cfg3a": ["softmax_cfg3a"],
             "fused_softmax_fwd_bwd_cfg3a": ["softmax_cfg3a"],
         }

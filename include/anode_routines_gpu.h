@@ -250,6 +250,9 @@ void anode_gpu_softmax_cat_nll_fused_packed_f32(uint32_t dim0, uint32_t dim1, co
 void anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, const float *dy, float *softmax, float *nll, float *dx, ANODE_LAUNCH_TAIL);
 /* softmax_nd and softmax_nd_cat_nll in one pass over x; writes the same softmax and nll as the two entry points. */
 void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, float *softmax, float *nll, ANODE_LAUNCH_TAIL);
+/* The same and the backward pass for a dy known before the forward pass, in one launch: softmax, nll and dx as
+ * softmax_nd, softmax_nd_cat_nll and softmax_nd_cat_nll_bwd write them (softmax.cu:227-334), bit for bit. */
+void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, const float *dy, float *softmax, float *nll, float *dx, ANODE_LAUNCH_TAIL);
 /* Running statistics: y <- fma(rate, x - y, y) (the semantics of anode's online_average, tests/test_gpu.rs:561-593). */
 void anode_gpu_online_average_packed_f32(uint32_t len, float rate, const float *x, float *y, ANODE_LAUNCH_TAIL);
 /* Device form of the host rule src/utils/mod.rs:31-41 per row of a [dim0 (fastest), dim1] array: first index of the

@@ -184,7 +184,8 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
         assert_bit_exact(host(dx_fa), host(dx_sa), "fused accumulate dx vs sequence")
 
 
-@pytest.mark.parametrize("P,C,N", [(64, 19, 2), (2048, 19, 2), (5, 3, 4), (1, 10, 6), (16, 32, 2), (8, 40, 3), (100, 1, 3)])
+@pytest.mark.parametrize("P,C,N", [(64, 19, 2), (2048, 19, 2), (5, 3, 4), (1, 10, 6), (16, 32, 2), (8, 40, 3), (100, 1, 3),
+                                   (1300, 19, 3), (516, 24, 2), (1028, 2, 3), (12, 7, 5)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N
@@ -200,6 +201,17 @@ def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
         assert_bit_exact(host(p2), host(p1), "fused softmax")
         assert_bit_exact(host(nll2), host(nll1), "fused nll")
         assert_close(host(p2), oracle.softmax_nd(P, C, N, x, f64=True), "fused softmax vs fp64", abs_floor=1e-30)
+        # forward and backward in one launch: the bits of the three launches
+        dy = g.standard_normal(P * N).astype(F32)
+        dx1 = empty(n, offset=offset)
+        call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dev(dy, offset), p1, dev(lab, offset), dx1)
+        p3, nll3, dx3 = empty(n, offset=offset), empty(P * N, offset=offset), empty(n, offset=offset)
+        call("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", P, C, N, dev(x, offset), dev(lab, offset),
+             dev(dy, offset), p3, nll3, dx3)
+        assert_bit_exact(host(p3), host(p1), "fwd+bwd fused softmax")
+        assert_bit_exact(host(nll3), host(nll1), "fwd+bwd fused nll")
+        assert_bit_exact(host(dx3), host(dx1), "fwd+bwd fused dx")
+        assert_bit_exact(host(dx3), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, host(p1), lab), "fwd+bwd fused dx vs oracle")
 
 
 ROW_FUSED_SHAPES = [(1, 5), (2, 7), (10, 32), (19, 513), (32, 600), (33, 9), (64, 300), (65, 3), (100, 17), (256, 5),
