@@ -82,108 +82,95 @@ __device__ inline float exp_nonpos(float d) {
   const float e = __builtin_amdgcn_exp2f(t);
   return fmaf(e, r * kLn2, e);
 }
-// K <= 64.  G = lanes per row (power of two >= K), log2g its logarithm.
-__global__ __launch_bounds__(kBlock) void softmax_row_subwave_kernel(uint32_t K, uint32_t R, uint32_t log2g,
-                                                                     const float *__restrict__ x,
-                                                                     float *__restrict__ y, RowNll nl) {
-  const uint32_t G = 1u << log2g;
-  const uint32_t rows_per_wave = uint32_t(kWave) >> log2g;
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t sub = lane >> log2g;
-  const uint32_t k = lane & (G - 1);
-  const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) / kWave;
-  const uint32_t n_waves = gridDim.x * (kBlock / kWave);
-  // the loop bound depends on the wave only, so all 64 lanes reach every shuffle
-  for (uint64_t r0 = uint64_t(wave) * rows_per_wave; r0 < R; r0 += uint64_t(n_waves) * rows_per_wave) {
-    const uint64_t r = r0 + sub;
-    const bool valid = (k < K) && (r < R);
-    const size_t idx = size_t(r) * K + k;
-    const float v = valid ? x[idx] : kNegInf;
-    const float m = group_max(v, int(G));
-    const float z = valid ? exp_nonpos(v - m) : 0.0f;
-    const float s = group_sum(z, int(G));
-    if (valid) {
-      const float pr = z * (1.0f / s);  // one correctly rounded reciprocal per row
-      y[idx] = pr;
-      if (nl.on()) nl.emit(r, K, nl.label(r), k, pr);
-    }
-  }
-}
-
-// K <= KMAX <= 32: one thread per row.  A workgroup takes 256 consecutive rows, which are 256*K contiguous floats:
-// they are copied to LDS as they lie in memory, 16 bytes per lane, each thread normalises its row in registers, and
-// the tile goes back the same way.  No cross-lane traffic at all, which is what bounds the lane-group kernel below
-// for short rows.  A thread walks its row from element (row number mod K) on, wrapping round: with every thread
-// starting at element 0 the lanes of a wave would meet in the same LDS banks whenever K is even (all 32 in one bank
-// for K = 32).  The sum of a row is therefore taken in an order that depends on the row number, and on nothing else.
-template <int KMAX, int NT>
-__global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, FastDiv div_k, int vec,
+// K <= 32 * G: G = 1, 2, 4 or 8 lanes per row, up to KMAX <= 32 values per lane.  A workgroup takes 256 / G
+// consecutive rows, which are contiguous floats: they are copied to LDS as they lie in memory, 16 bytes per lane,
+// each lane group normalises its row in registers, and the tile goes back the same way, so every global access
+// is a full-width coalesced one whatever K is.  Lane l of a group holds the classes l, l + G, l + 2G, ... and walks
+// them from the `rot * row`-th on, wrapping round: the host picks rot (0 to 3) so that the lanes of a wave meet in
+// different LDS banks (rows K floats apart would otherwise share banks whenever K / G is even).  The sum of a row
+// is therefore taken in an order that depends on K and on the row number, and on nothing else.
+template <int KMAX, int LOG2G, int NT>
+__global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uint32_t R, uint32_t rot,
+                                                                 FastDiv div_kj, int vec,
                                                                  const float *__restrict__ x,
                                                                  float *__restrict__ y, RowNll nl) {
-  extern __shared__ __align__(16) float tile[];  // kBlock * K floats
+  extern __shared__ __align__(16) float tile[];  // (kBlock >> LOG2G) * K floats, at most 32 KiB
   f32x4 *tile4 = reinterpret_cast<f32x4 *>(tile);
-  for (uint64_t r0 = uint64_t(blockIdx.x) * kBlock; r0 < R; r0 += uint64_t(gridDim.x) * kBlock) {
-    const uint32_t rows = (R - r0 < uint64_t(kBlock)) ? uint32_t(R - r0) : uint32_t(kBlock);
+  constexpr uint32_t G = 1u << LOG2G;
+  constexpr uint32_t rows_per_block = uint32_t(kBlock) >> LOG2G;
+  const uint32_t KJ = div_kj.d;                    // ceil(K / G): values a lane may hold
+  const uint32_t local = threadIdx.x >> LOG2G;     // row of the tile
+  const uint32_t l = threadIdx.x & (G - 1u);       // lane of the row's group
+  uint32_t q0, first;
+  div_kj.divmod(local * rot, q0, first);           // where this row's walk starts
+  for (uint64_t r0 = uint64_t(blockIdx.x) * rows_per_block; r0 < R; r0 += uint64_t(gridDim.x) * rows_per_block) {
+    const uint32_t rows = (R - r0 < uint64_t(rows_per_block)) ? uint32_t(R - r0) : rows_per_block;
     const uint32_t n = rows * K;
     const float *xt = x + r0 * K;
     float *yt = y + r0 * K;
-    const uint32_t n4 = vec ? n / 4u : 0u;  // the tile starts 1024*K bytes into an aligned array: 16-byte aligned
+    // (the tile starts a multiple of 32 rows into an aligned array: 16-byte aligned)
+    const uint32_t n4 = vec ? n / 4u : 0u;
     // the row's label and upstream gradient are requested together with the tile
-    const uint64_t r = r0 + threadIdx.x;
-    const bool mine = threadIdx.x < rows;
+    const uint64_t r = r0 + local;
+    const bool mine = local < rows;  // the same for all lanes of a row's group
     const uint32_t label = (mine && nl.on()) ? nl.label(r) : 0u;
     const float dyr = (mine && nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
     for (uint32_t g = threadIdx.x; g < n4; g += kBlock) tile4[g] = reinterpret_cast<const f32x4 *>(xt)[g];
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) tile[e] = xt[e];
     __syncthreads();
-    float *row = tile + threadIdx.x * K;
-    uint32_t q0, first;
-    div_k.divmod(uint32_t(r), q0, first);  // first = row number mod K (r < 2^32: K * R fits 32 bits)
+    float *row = tile + local * K + l;  // this lane's classes are row[0], row[G], row[2G], ...
     float v[KMAX];
-    if (mine) {
+    if (mine) {  // whole lane groups take this branch or skip it, so the exchanges below stay inside active lanes
       float m = kNegInf;
       uint32_t at = first;
 #pragma unroll
-      for (int k = 0; k < KMAX; ++k) {
-        if (uint32_t(k) < K) {
-          v[k] = row[at];
-          m = fmaxf(m, v[k]);
-          at = (at + 1u == K) ? 0u : at + 1u;
+      for (int j = 0; j < KMAX; ++j) {
+        if (uint32_t(j) < KJ) {
+          v[j] = (G == 1u || l + (at << LOG2G) < K) ? row[at << LOG2G] : kNegInf;
+          m = fmaxf(m, v[j]);
+          at = (at + 1u == KJ) ? 0u : at + 1u;
         }
       }
+      if (G > 1u) m = group_max(m, int(G));
       float sum = 0.0f;
 #pragma unroll
-      for (int k = 0; k < KMAX; ++k) {
-        if (uint32_t(k) < K) {
-          v[k] = exp_nonpos(v[k] - m);
-          sum += v[k];
+      for (int j = 0; j < KMAX; ++j) {
+        if (uint32_t(j) < KJ) {
+          v[j] = exp_nonpos(v[j] - m);  // a slot past the row's end holds -inf and adds 0
+          sum += v[j];
         }
       }
+      if (G > 1u) sum = group_sum(sum, int(G));
       const float rsum = 1.0f / sum;  // one correctly rounded reciprocal per row
       at = first;
 #pragma unroll
-      for (int k = 0; k < KMAX; ++k) {
-        if (uint32_t(k) < K) {
-          v[k] = v[k] * rsum;
-          row[at] = v[k];
-          at = (at + 1u == K) ? 0u : at + 1u;
+      for (int j = 0; j < KMAX; ++j) {
+        if (uint32_t(j) < KJ) {
+          v[j] = v[j] * rsum;
+          if (G == 1u || l + (at << LOG2G) < K) row[at << LOG2G] = v[j];
+          at = (at + 1u == KJ) ? 0u : at + 1u;
         }
       }
-      if (nl.on()) nl.emit_nll(r, K, label, label < K ? label : 0u, label < K ? row[label] : 0.0f);
     }
-    __syncthreads();
+    if (G > 1u) __syncthreads();  // the label's probability may have been written by another wave's lane
+    if (mine && l == 0u && nl.on()) {
+      const float *whole = tile + local * K;
+      nl.emit_nll(r, K, label, label < K ? label : 0u, label < K ? whole[label] : 0.0f);
+    }
+    if (G == 1u) __syncthreads();
     for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, tile4[g]);
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) yt[e] = tile[e];
     __syncthreads();  // the tile is overwritten below, or by the next pass
     if (nl.on() && nl.dx != nullptr) {
-      // the gradient takes the same way out: each thread turns its row into dy * (p - onehot) in place
+      // the gradient takes the same way out: each lane turns its classes into dy * (p - onehot) in place
       if (mine) {
         uint32_t at = first;
 #pragma unroll
-        for (int k = 0; k < KMAX; ++k) {
-          if (uint32_t(k) < K) {
-            row[at] = RowNll::grad(dyr, label, at, v[k]);
-            at = (at + 1u == K) ? 0u : at + 1u;
+        for (int j = 0; j < KMAX; ++j) {
+          if (uint32_t(j) < KJ) {
+            const uint32_t k = l + (at << LOG2G);
+            if (G == 1u || k < K) row[at << LOG2G] = RowNll::grad(dyr, label, k, v[j]);
+            at = (at + 1u == KJ) ? 0u : at + 1u;
           }
         }
       }
@@ -196,7 +183,30 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
   }
 }
 
-// 64 < K <= 64 * VPL: one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
+// The rotation (0 to 3 places per row) that spreads the first LDS access of a wave's 32-lane halves over most banks.
+uint32_t pick_row_rotation(uint32_t K, uint32_t log2g) {
+  const uint32_t G = 1u << log2g, KJ = (K + G - 1) / G;
+  uint32_t best = 0, best_worst = ~0u;
+  for (uint32_t rot = 0; rot < 4; ++rot) {
+    uint32_t hits[32] = {0};
+    uint32_t worst = 0;
+    for (uint32_t t = 0; t < 32; ++t) {  // 32 lanes are served per cycle
+      const uint32_t local = t >> log2g, l = t & (G - 1u);
+      const uint32_t at = (local * rot) % KJ;
+      uint32_t k = l + G * at;
+      if (k >= K) k = l;  // such a lane sits the access out; count it where its next one goes
+      const uint32_t bank = (local * K + k) % 32u;
+      if (++hits[bank] > worst) worst = hits[bank];
+    }
+    if (worst < best_worst) {
+      best_worst = worst;
+      best = rot;
+    }
+  }
+  return best;
+}
+
+// 208 < K <= 64 * VPL: one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
 // of 4, aligned arrays) and a lane owns groups of four consecutive classes; otherwise lane l owns k = l, l+64, ...
 template <int VPL, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
@@ -425,31 +435,47 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   const uint32_t max_blocks = 1u << 24;
   constexpr uint32_t kWavesPerBlock = kBlock / kWave;
   const int nt = stream_policy(size_t(K) * R * sizeof(float), tuning().nontemporal);  // logits in, probabilities out: both streamed
-  if (K <= 32) {
-    uint32_t blocks = (R + kBlock - 1) / kBlock;
+  if (K <= 208) {
+    // 1, 2, 4 or 8 lanes per row, at most 32 values per lane; the tile of 256 / G rows is at most 32 KiB.
+    // (From 209 columns on the wave-per-row kernel below keeps enough of its 64 lanes busy to be faster:
+    // 6.1 TB/s against 4.5 at 256 columns, 4.3 against 4.7 at 200.)
+    uint32_t log2g = 0;
+    while ((32u << log2g) < K) ++log2g;
+    const uint32_t G = 1u << log2g, KJ = (K + G - 1) / G;
+    const uint32_t rows_per_block = uint32_t(kBlock) >> log2g;
+    uint32_t blocks = (R + rows_per_block - 1) / rows_per_block;
     if (blocks > max_blocks) blocks = max_blocks;
-    const size_t lds_bytes = size_t(kBlock) * K * sizeof(float);
-    const FastDiv div_k(K);
+    const size_t lds_bytes = size_t(rows_per_block) * K * sizeof(float);
+    const FastDiv div_kj(KJ);
+    const uint32_t rot = pick_row_rotation(K, log2g);
     const int vec = (aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx))) ? 1 : 0;
     with_stream_policy(nt & kNtStore, [&](auto policy) {
       constexpr int NT = decltype(policy)::value;
-      if (K <= 4) {
-        softmax_row_lds_kernel<4, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
-      } else if (K <= 8) {
-        softmax_row_lds_kernel<8, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
-      } else if (K <= 16) {
-        softmax_row_lds_kernel<16, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
+      auto launch = [&](auto kmax, auto lg) {
+        softmax_row_lds_kernel<decltype(kmax)::value, decltype(lg)::value, NT>
+            <<<blocks, kBlock, lds_bytes, s>>>(K, R, rot, div_kj, vec, x, y, nl);
+      };
+      auto with_kmax = [&](auto lg) {
+        if (KJ <= 4) {
+          launch(std::integral_constant<int, 4>{}, lg);
+        } else if (KJ <= 8) {
+          launch(std::integral_constant<int, 8>{}, lg);
+        } else if (KJ <= 16) {
+          launch(std::integral_constant<int, 16>{}, lg);
+        } else {
+          launch(std::integral_constant<int, 32>{}, lg);
+        }
+      };
+      if (log2g == 0) {
+        with_kmax(std::integral_constant<int, 0>{});
+      } else if (log2g == 1) {
+        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 1>{});  // 32 < K <= 64: 17 to 32 values
+      } else if (log2g == 2) {
+        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 2>{});
       } else {
-        softmax_row_lds_kernel<32, NT><<<blocks, kBlock, lds_bytes, s>>>(K, R, div_k, vec, x, y, nl);
+        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 3>{});
       }
     });
-  } else if (K <= 64) {
-    uint32_t log2g = 0;
-    while ((1u << log2g) < K) ++log2g;
-    const uint32_t rows_per_block = kWavesPerBlock * (64u >> log2g);
-    uint32_t blocks = (R + rows_per_block - 1) / rows_per_block;
-    if (blocks > max_blocks) blocks = max_blocks;
-    softmax_row_subwave_kernel<<<blocks, kBlock, 0, s>>>(K, R, log2g, x, y, nl);
   } else if (K <= 2048) {
     uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > max_blocks) blocks = max_blocks;

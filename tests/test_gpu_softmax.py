@@ -48,6 +48,8 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (128, 5), (129, 4), (1000, 256), (1024, 3), (1025, 2), (2048, 2), (2049, 3), (5000, 2), (40000, 1),
               # several 256-row tiles of the thread-per-row kernel, ragged last tile, even and odd K
               (10, 4000), (7, 777), (32, 600), (16, 257), (4, 1025), (5, 256), (31, 1023),
+              # either side of the switch from lane groups over an LDS tile to one wave per row, 2 to 8 lanes per row
+              (208, 70), (209, 70), (212, 33), (40, 1000), (96, 300), (130, 77), (200, 50),
               # the limits of the workgroup-per-row register kernel
               (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1)]
 
