@@ -602,17 +602,30 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
   p = r * uint32_t(W);
 }
 
-__device__ inline float pair_swap(float v) { return __shfl_xor(v, 1, kWave); }
-__device__ inline f32x4 pair_swap(f32x4 v) {
-  return f32x4{__shfl_xor(v.x, 1, kWave), __shfl_xor(v.y, 1, kWave), __shfl_xor(v.z, 1, kWave), __shfl_xor(v.w, 1, kWave)};
+// Marks the point from which a loaded value is known to have arrived.  The streaming stores are inline assembly,
+// which the compiler's wait-count bookkeeping does not see: where the first use of an earlier load sits in a
+// conditional block after such stores, the wait it inserts there (for "the load") also waits for every store
+// issued since, one store at a time.  Using the value once before the stores begin removes those waits.
+// (The memory clobber keeps the loads written before the mark before it, and those after it after it.)
+__device__ inline void arrived(float v) { asm volatile("" ::"v"(v) : "memory"); }
+__device__ inline void arrived(uint32_t v) { asm volatile("" ::"v"(v) : "memory"); }
+__device__ inline void arrived(f32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
+__device__ inline void arrived(u32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
+__device__ inline void issue_order_fence() { asm volatile("" ::: "memory"); }
+
+// the value held by the lane whose number differs in the bits of `off`
+__device__ inline float lane_swap(float v, int off) { return __shfl_xor(v, off, kWave); }
+__device__ inline f32x4 lane_swap(f32x4 v, int off) {
+  return f32x4{__shfl_xor(v.x, off, kWave), __shfl_xor(v.y, off, kWave), __shfl_xor(v.z, off, kWave),
+               __shfl_xor(v.w, off, kWave)};
 }
 
-// C <= CMAX: the pixel's classes stay in registers, x is read once.  SPLIT lanes (1 or 2) share a group of W
-// pixels: lane h of the pair holds classes h, h + SPLIT, ... and the pair's maxima and sums meet through one lane
-// exchange each.  Two lanes per group halve a thread's state (ten 16-byte loads in flight instead of nineteen at
-// C = 19) and measured 112 us against 120 us at [512K, 19, 8]; four or eight lanes are slower again (118, 122 us:
-// a load instruction then covers several short runs).  A lane adds its exponentials in class order, the pair's sums
-// are added last; the normalisation multiplies by one correctly rounded reciprocal per pixel.  With NLL the label
+// C <= CMAX: the pixel's classes stay in registers, x is read once.  SPLIT lanes (1, 2 or 8) share a group of W
+// pixels: lane h of the group holds classes h, h + SPLIT, ... and the group's maxima and sums meet through lane
+// exchanges.  Two lanes per group halve a thread's state (ten 16-byte loads in flight instead of nineteen at
+// C = 19) and measured 112 us against 120 us at [512K, 19, 8]; four or eight lanes are slower there (118, 122 us:
+// a load instruction then covers several short runs), but they are what keeps 33 to 256 classes in registers.
+// A lane adds its exponentials in class order, the group's sums are added last; the normalisation multiplies by one correctly rounded reciprocal per pixel.  With NLL the label
 // gather is fused: nll = -log(the stored probability of the label), NaN when the label is out of range, exactly
 // what the separate gather returns.
 // With BWD the gradient of the summed loss for a dy known up front is written in the same pass:
@@ -636,18 +649,25 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     uint32_t p, n;
     pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
+    const size_t pix = size_t(p) + size_t(pg.P) * n;
+    // the labels and the upstream gradient are requested first, so that they are there when the classes are
+    U lab;
+    if (NLL) lab = *reinterpret_cast<const U *>(cat + pix);
+    V d;
+    if (BWD) d = *reinterpret_cast<const V *>(dy + pix);
+    if (NLL) issue_order_fence();
+    // Every slot is loaded, a slot past the last class from the last class's plane again (and set to -inf below):
+    // with a branch round each load the compiler waits for the previous load before it issues the next one.
     V v[H];
 #pragma unroll
     for (int i = 0; i < H; ++i) {
       const uint32_t k = uint32_t(i) * SPLIT + h;
-      if (k < pg.C) v[i] = load_stream<NT>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
+      const uint32_t kk = k < pg.C ? k : pg.C - 1u;
+      v[i] = load_stream<NT>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * kk));
     }
-    const size_t pix = size_t(p) + size_t(pg.P) * n;
-    U lab;
-    if (NLL) lab = *reinterpret_cast<const U *>(cat + pix);
-    V d;
+    if (NLL) arrived(lab);
     if (BWD) {
-      d = *reinterpret_cast<const V *>(dy + pix);
+      arrived(d);
       if (pg.ignore) {
 #pragma unroll
         for (int w = 0; w < W; ++w) {
@@ -658,18 +678,21 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     V m = PixVec<V>::splat(kNegInf);
 #pragma unroll
     for (int i = 0; i < H; ++i) {
-      if (uint32_t(i) * SPLIT + h < pg.C) m = vmax(m, v[i]);
+      if (uint32_t(i) * SPLIT + h >= pg.C) v[i] = PixVec<V>::splat(kNegInf);
+      m = vmax(m, v[i]);
     }
-    if (SPLIT == 2) m = vmax(m, pair_swap(m));
+#pragma unroll
+    for (int off = 1; off < SPLIT; off <<= 1) m = vmax(m, lane_swap(m, off));
     V s = PixVec<V>::splat(0.0f);
 #pragma unroll
     for (int i = 0; i < H; ++i) {
-      if (uint32_t(i) * SPLIT + h < pg.C) {
-        v[i] = vexp(v[i] - m);
-        s += v[i];
-      }
+      // a slot past the last class holds -inf and adds exp(-inf - m) = 0 (NaN only where m is -inf or NaN, and
+      // then the pixel's own classes give NaN as well)
+      v[i] = vexp(v[i] - m);
+      s += v[i];
     }
-    if (SPLIT == 2) s += pair_swap(s);  // a + b == b + a: both lanes hold the same sum
+#pragma unroll
+    for (int off = 1; off < SPLIT; off <<= 1) s += lane_swap(s, off);  // a + b == b + a: every lane holds the same sum
     const V inv = vrcp(s);
 #pragma unroll
     for (int i = 0; i < H; ++i) {
@@ -697,16 +720,13 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
       for (int i = 0; i < H; ++i) {
 #pragma unroll
         for (int w = 0; w < W; ++w) {
-          if (lane_get_u(lab, w) / uint32_t(SPLIT) == uint32_t(i)) lane_set<V>(pick, w, lane_get<V>(v[i], w));
+          const uint32_t lb = lane_get_u(lab, w);
+          if (lb / uint32_t(SPLIT) == uint32_t(i) && lb % uint32_t(SPLIT) == h) lane_set<V>(pick, w, lane_get<V>(v[i], w));
         }
       }
-      if (SPLIT == 2) {
-        const V other = pair_swap(pick);
+      // one lane of the group holds the label's exponential, the others hold 0: the sum hands it to all of them
 #pragma unroll
-        for (int w = 0; w < W; ++w) {
-          if (lane_get_u(lab, w) % 2u != h) lane_set<V>(pick, w, lane_get<V>(other, w));
-        }
-      }
+      for (int off = 1; off < SPLIT; off <<= 1) pick += lane_swap(pick, off);
       if (h == 0) {
         V out;
 #pragma unroll
@@ -720,24 +740,61 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
   }
 }
 
-// any C: online max/sum pass over the classes, then a normalising pass
+// any C: one pass over the classes that keeps a running maximum and a running sum of exponentials, eight planes
+// requested at a time, then a normalising pass (x is read twice; the reference reads it three times).  A block of
+// planes is folded into (its maximum, the sum of its exponentials about that maximum) and merged with the running
+// pair by online_merge(), which also keeps -inf planes from turning into NaN.
 template <typename V>
 __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                    float *__restrict__ y) {
   constexpr int W = PixVec<V>::W;
+  constexpr int U = 8;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
     pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     V m = PixVec<V>::splat(kNegInf);
-    for (uint32_t k = 0; k < pg.C; ++k) m = vmax(m, *reinterpret_cast<const V *>(x + base + size_t(pg.P) * k));
     V s = PixVec<V>::splat(0.0f);
-    for (uint32_t k = 0; k < pg.C; ++k) s += vexp(*reinterpret_cast<const V *>(x + base + size_t(pg.P) * k) - m);
+    for (uint32_t k0 = 0; k0 < pg.C; k0 += U) {
+      V v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {  // a slot past the last class reads the last class again and is set to -inf
+        const uint32_t k = k0 + uint32_t(u);
+        v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
+      }
+      V bm = PixVec<V>::splat(kNegInf);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (k0 + uint32_t(u) >= pg.C) v[u] = PixVec<V>::splat(kNegInf);
+        bm = vmax(bm, v[u]);
+      }
+      V bs = PixVec<V>::splat(0.0f);
+#pragma unroll
+      for (int u = 0; u < U; ++u) bs += vexp(v[u] - bm);
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        float mw = lane_get<V>(m, w), sw = lane_get<V>(s, w);
+        const float bmw = lane_get<V>(bm, w);
+        // a block of -inf planes has seen nothing: its sum, exp(-inf - -inf) = NaN, is not a sum
+        online_merge(mw, sw, bmw, bmw == kNegInf ? 0.0f : lane_get<V>(bs, w));
+        lane_set<V>(m, w, mw);
+        lane_set<V>(s, w, sw);
+      }
+    }
     const V inv = vrcp(s);
-    for (uint32_t k = 0; k < pg.C; ++k) {
-      const V z = vexp(*reinterpret_cast<const V *>(x + base + size_t(pg.P) * k) - m);
-      *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = z * inv;
+    for (uint32_t k0 = 0; k0 < pg.C; k0 += U) {
+      V v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t k = k0 + uint32_t(u);
+        v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t k = k0 + uint32_t(u);
+        if (k < pg.C) *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = vexp(v[u] - m) * inv;
+      }
     }
   }
 }
@@ -829,7 +886,7 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore
 // one pixel group per thread: the hardware dispatcher walks the array in order
 uint32_t pixel_blocks(uint32_t total_groups) { return stream_grid(total_groups, 1); }
 
-// C <= 32 only.  The 16-byte form runs two lanes per pixel group.
+// C <= 32, or C <= 256 in the 16-byte form, which runs two, four or eight lanes per pixel group.
 template <typename V, bool NLL, int NT, bool BWD = false>
 void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
                               float *nll, hipStream_t s, const float *dy = nullptr, float *dx = nullptr,
@@ -837,6 +894,23 @@ void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x
   constexpr int SPLIT = PixVec<V>::W == 4 ? 2 : 1;
   PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W, ignore);
   pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
+  if constexpr (PixVec<V>::W == 4) {
+    // more classes: eight lanes per pixel group, 8, 16 or 32 sixteen-byte values per lane
+    if (C > 128) {
+      softmax_nd_reg_kernel<256, V, NLL, NT, 8, BWD>
+          <<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
+      return;
+    } else if (C > 64) {
+      softmax_nd_reg_kernel<128, V, NLL, NT, 8, BWD>
+          <<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
+      return;
+    } else if (C > 32) {
+      // (eight lanes of 8 values, 106 to 123 registers, rather than four lanes of 16, 164 to 195)
+      softmax_nd_reg_kernel<64, V, NLL, NT, 8, BWD>
+          <<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
+      return;
+    }
+  }
   const uint32_t blocks = stream_grid(uint64_t(pg.total_groups) * SPLIT, 1);
   if (C <= 4) {
     softmax_nd_reg_kernel<4, V, NLL, NT, SPLIT, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
@@ -870,7 +944,7 @@ void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, f
 
 template <typename V>
 void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, hipStream_t s) {
-  if (C <= 32) {
+  if (C <= 32 || (PixVec<V>::W == 4 && C <= 256)) {
     launch_softmax_nd_reg<V, false>(P, C, N, x, y, nullptr, nullptr, s);
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
@@ -888,8 +962,8 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
-  if (C > 32 && C <= 128) {
-    // too many classes for four pixels per thread: one pixel per thread keeps
+  if (!vec && C > 32 && C <= 128) {
+    // too many classes for four pixels per thread without 16-byte accesses: one pixel per thread keeps
     // the row in registers and is still coalesced across the wave
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
     const uint32_t blocks = pixel_blocks(pg.total_groups);
@@ -1054,9 +1128,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
-  } else if (dim0 <= 32) {
+  } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
+                              aligned16(nll);
+             dim0 <= 32 || (vec && dim0 <= 256)) {
     hipStream_t s = as_stream(stream);
-    const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) && aligned16(nll);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
     } else {
@@ -1082,10 +1157,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
-  } else if (dim0 <= 32) {
+  } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
+                              aligned16(nll) && aligned16(dy) && aligned16(dx);
+             dim0 <= 32 || (vec && dim0 <= 256)) {
     hipStream_t s = as_stream(stream);
-    const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
-                     aligned16(nll) && aligned16(dy) && aligned16(dx);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
     } else {

@@ -185,7 +185,8 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
 
 
 @pytest.mark.parametrize("P,C,N", [(64, 19, 2), (2048, 19, 2), (5, 3, 4), (1, 10, 6), (16, 32, 2), (8, 40, 3), (100, 1, 3),
-                                   (1300, 19, 3), (516, 24, 2), (1028, 2, 3), (12, 7, 5)])
+                                   (1300, 19, 3), (516, 24, 2), (1028, 2, 3), (12, 7, 5),
+                                   (20, 48, 3), (24, 129, 2), (16, 200, 2), (8, 256, 3), (8, 300, 2), (520, 40, 2)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

@@ -134,7 +134,10 @@ def test_softmax_cat_nll_and_bwd_rows(oracle, K, R):
 ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100, 1, 3), (36, 4, 2), (40, 8, 3),
              (28, 16, 2), (12, 24, 2), (16, 32, 2), (8, 33, 2), (8, 64, 3), (6, 100, 2), (4, 130, 2), (7, 40, 3),
              # several waves of pixel groups with a ragged last wave, few and many classes
-             (1300, 19, 3), (516, 32, 5), (1028, 2, 3)]
+             (1300, 19, 3), (516, 32, 5), (1028, 2, 3),
+             # eight lanes per pixel group (33 to 256 classes with 16-byte accesses), and the streamed kernel beyond
+             (20, 48, 3), (20, 64, 2), (24, 65, 2), (24, 128, 2), (24, 129, 2), (16, 200, 2), (8, 256, 3), (520, 40, 2),
+             (8, 300, 2), (5, 257, 3), (64, 1000, 2), (7, 300, 2)]
 
 
 @pytest.mark.parametrize("P,C,N", ND_SHAPES)
@@ -172,9 +175,10 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
         assert_bit_exact(host(dxa), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, dx_in=old), "nd bwd acc vs fp32")
 
 
-@pytest.mark.parametrize("C", [3, 19, 40, 200])
+@pytest.mark.parametrize("C", [3, 19, 40, 100, 200, 300])
 def test_softmax_nd_special_values(oracle, C):
-    # register-resident (C <= 32, C <= 128) and streaming (C > 128) kernels: -inf entries get probability 0, a NaN
+    # register-resident (2 or 8 lanes per pixel group up to 256 classes; one pixel per thread without 16-byte
+    # accesses up to 128) and streaming kernels: -inf entries get probability 0, a NaN
     # poisons its pixel only, a pixel of +-1e30 and one of large equal values do not overflow, widely spread logits
     # keep their small probabilities to the relative bar
     P, N = 8, 2
