@@ -117,12 +117,14 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_chunk_kernel(ReducePlan pl
       V va[U], vb[U], vc[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
+        // Every slot is loaded, a slot past the tile's end from the tile's last group again (and left out of the
+        // sums below): with a branch round each load the compiler waits for the previous load before it issues
+        // the next one.  (LG >= 1: a tile is never empty.)
         const uint32_t j = jb + uint32_t(u) * kBlock + threadIdx.x;
-        if (j < LG) {
-          va[u] = load_stream<NT>(&pa[j]);
-          if (Op::NIN >= 2) vb[u] = load_stream<NT>(&pb[j]);
-          if (Op::NIN >= 3) vc[u] = load_stream<NT>(&pc[j]);
-        }
+        const uint32_t jc = j < LG ? j : LG - 1u;
+        va[u] = load_stream<NT>(&pa[jc]);
+        if (Op::NIN >= 2) vb[u] = load_stream<NT>(&pb[jc]);
+        if (Op::NIN >= 3) vc[u] = load_stream<NT>(&pc[jc]);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -201,17 +203,20 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
     V va[STAGES][G], vb[STAGES][G], vc[STAGES][G];
 #pragma unroll
     for (int sg = 0; sg < STAGES; ++sg) {
-      if (n + uint32_t(sg) < n1) {
-        const V *pa = reinterpret_cast<const V *>(a + (size_t(n + sg) * CS + p0));
-        const V *pb = reinterpret_cast<const V *>(b + (size_t(n + sg) * CS + p0));
-        const V *pc = reinterpret_cast<const V *>(c3 + (size_t(n + sg) * CS + p0));
+      {
+        // unconditional, as in the chunk kernel: a stage past the last sample reads the last sample again, a slot
+        // past the tile's end the tile's last group; neither is added below
+        const uint32_t ns = (n + uint32_t(sg) < n1) ? n + uint32_t(sg) : n1 - 1u;
+        const V *pa = reinterpret_cast<const V *>(a + (size_t(ns) * CS + p0));
+        const V *pb = reinterpret_cast<const V *>(b + (size_t(ns) * CS + p0));
+        const V *pc = reinterpret_cast<const V *>(c3 + (size_t(ns) * CS + p0));
 #pragma unroll
         for (int i = 0; i < G; ++i) {
-          if (valid[i]) {
-            va[sg][i] = load_stream<NT>(&pa[threadIdx.x + uint32_t(i) * kBlock]);
-            if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[threadIdx.x + uint32_t(i) * kBlock]);
-            if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[threadIdx.x + uint32_t(i) * kBlock]);
-          }
+          const uint32_t j = threadIdx.x + uint32_t(i) * kBlock;
+          const uint32_t jc = valid[i] ? j : LG - 1u;
+          va[sg][i] = load_stream<NT>(&pa[jc]);
+          if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[jc]);
+          if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[jc]);
         }
       }
     }
