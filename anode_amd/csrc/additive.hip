@@ -69,12 +69,15 @@ __global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t n_group
   uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
   const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // first group = first output dword
-  f32x4 v[4];
+  f32x4 v[4] = {};
+  if (n_groups != 0u) {  // (fewer than four elements: only the tail below has work)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const uint64_t g = wave_first + uint32_t(j) * kWave + lane;
-    v[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    if (g < n_groups) v[j] = load_stream<kNtLoad>(&x4[g]);
+    for (int j = 0; j < 4; ++j) {
+      // unconditional (a group past the end reads the last group again; its code is never stored): with a branch
+      // round each load the compiler waits for the previous load before it issues the next one
+      const uint64_t g = wave_first + uint32_t(j) * kWave + lane;
+      v[j] = load_stream<kNtLoad>(&x4[g < n_groups ? g : uint64_t(n_groups - 1u)]);
+    }
   }
   uint32_t d[4];
 #pragma unroll
