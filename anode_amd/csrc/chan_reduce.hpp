@@ -213,10 +213,20 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_whole_kernel(ReducePlan pl
 #pragma unroll
         for (int i = 0; i < G; ++i) {
           const uint32_t j = threadIdx.x + uint32_t(i) * kBlock;
-          const uint32_t jc = valid[i] ? j : LG - 1u;
-          va[sg][i] = load_stream<NT>(&pa[jc]);
-          if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[jc]);
-          if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[jc]);
+          if (W == 1) {
+            // element-aligned arrays (thirty-two 4-byte loads per batch): here the branches cost less than the extra
+            // loads do, batch_norm_bwd_var at [1025, 64, 1023] 5.6 TB/s against 4.4
+            if (valid[i]) {
+              va[sg][i] = load_stream<NT>(&pa[j]);
+              if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[j]);
+              if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[j]);
+            }
+          } else {
+            const uint32_t jc = valid[i] ? j : LG - 1u;
+            va[sg][i] = load_stream<NT>(&pa[jc]);
+            if (Op::NIN >= 2) vb[sg][i] = load_stream<NT>(&pb[jc]);
+            if (Op::NIN >= 3) vc[sg][i] = load_stream<NT>(&pc[jc]);
+          }
         }
       }
     }
