@@ -19,6 +19,7 @@ SHAPES = [
     (49, 3, 5),       # C*S odd: element path
     (1, 37, 11),      # S == 1
     (1, 1000, 64),
+    (1, 512, 40), (2, 6, 33), (3, 8, 17), (1, 4, 16), (2, 64, 100), (3, 4, 15),   # channels shorter than a 16-byte group
     (2, 5, 3),
     (16, 300, 3),     # more channels than a tile may hold
     (7, 513, 2),
