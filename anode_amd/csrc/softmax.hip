@@ -853,19 +853,41 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
         if (lane_get_u(lab, w) >= pg.C) lane_set<V>(d, w, 0.0f);
       }
     }
-#pragma unroll 4
-    for (uint32_t k = 0; k < pg.C; ++k) {
-      const size_t off = base + size_t(pg.P) * k;
-      const V pr = load_stream<NT>(reinterpret_cast<const V *>(prob + off));
-      V old;
-      if (ACC) old = load_stream<NT>(reinterpret_cast<const V *>(dx + off));
-      V r;
+    // Four planes are requested together (a slot past the last class reads the last class again), then written:
+    // the streaming store is an ordering point for the compiler, so a plane-by-plane loop keeps one load in flight.
+    constexpr int B = 4;
+    V pr[B], old[B];
+    auto request = [&](uint32_t k0) {
 #pragma unroll
-      for (int w = 0; w < W; ++w) {
-        const float t = lane_get<V>(pr, w) - float(lane_get_u(lab, w) == k);
-        lane_set<V>(r, w, ACC ? fmaf(lane_get<V>(d, w), t, lane_get<V>(old, w)) : lane_get<V>(d, w) * t);
+      for (int u = 0; u < B; ++u) {
+        const uint32_t k = k0 + uint32_t(u) < pg.C ? k0 + uint32_t(u) : pg.C - 1u;
+        const size_t off = base + size_t(pg.P) * k;
+        pr[u] = load_stream<NT>(reinterpret_cast<const V *>(prob + off));
+        if (ACC) old[u] = load_stream<NT>(reinterpret_cast<const V *>(dx + off));
       }
-      store_stream<NT>(reinterpret_cast<V *>(dx + off), r);
+    };
+    auto write = [&](uint32_t k0) {
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        const uint32_t k = k0 + uint32_t(u);
+        if (k < pg.C) {
+          V r;
+#pragma unroll
+          for (int w = 0; w < W; ++w) {
+            const float t = lane_get<V>(pr[u], w) - float(lane_get_u(lab, w) == k);
+            lane_set<V>(r, w, ACC ? fmaf(lane_get<V>(d, w), t, lane_get<V>(old[u], w)) : lane_get<V>(d, w) * t);
+          }
+          store_stream<NT>(reinterpret_cast<V *>(dx + base + size_t(pg.P) * k), r);
+        }
+      }
+    };
+    request(0);
+    arrived(d);  // dy and the labels were requested first: known to be there before the first store is issued
+    arrived(lab);
+    write(0);
+    for (uint32_t k0 = uint32_t(B); k0 < pg.C; k0 += uint32_t(B)) {
+      request(k0);
+      write(k0);
     }
   }
 }
