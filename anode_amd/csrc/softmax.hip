@@ -913,6 +913,7 @@ template <typename V, bool NLL, int NT, bool BWD = false>
 void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
                               float *nll, hipStream_t s, const float *dy = nullptr, float *dx = nullptr,
                               bool ignore = false) {
+  // (the same lanes per group in every variant: the order of a pixel's sum, hence the bits of p, depends on it)
   constexpr int SPLIT = PixVec<V>::W == 4 ? 2 : 1;
   PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W, ignore);
   pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
