@@ -100,11 +100,12 @@ __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uin
     V va[UNROLL], vb[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
+      // unconditional (a slot past the end reads the last group again and is not stored): with a branch round
+      // each load the compiler waits for the previous load before it issues the next one
       const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) {
-        va[u] = load_stream<NT>(&a[g]);
-        vb[u] = (NIN == 2) ? load_stream<NT>(&b[g]) : va[u];
-      }
+      const uint64_t gc = g < n_groups ? g : uint64_t(n_groups) - 1u;
+      va[u] = load_stream<NT>(&a[gc]);
+      vb[u] = (NIN == 2) ? load_stream<NT>(&b[gc]) : va[u];
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -131,6 +132,8 @@ void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, co
   if (vec) {
     // one 16-byte group per thread: measured faster on MI355X than any unrolled persistent loop
     const uint32_t groups = len / 4, tail = len % 4;
+    // (Two or four groups per thread on a correspondingly smaller grid, all their loads in flight together, run at
+    // 6.1 TB/s against 6.65 for the copy of 822 MB arrays.)
     with_stream_policy(nt, [&](auto policy) {
       flat_map_kernel<f32x4, NIN, 1, decltype(policy)::value, Op>
           <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out);
