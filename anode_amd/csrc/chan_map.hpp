@@ -67,13 +67,14 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
     V va[UNROLL], vb[UNROLL], vc[UNROLL], vo[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
+      // unconditional (a slot past the end reads the last group again and is not stored): with a branch round
+      // each load the compiler waits for the previous load before it issues the next one
       const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) {
-        if (NIN >= 1) va[u] = load_stream<NT>(&a[g]);
-        if (NIN >= 2) vb[u] = load_stream<NT>(&b[g]);
-        if (NIN >= 3) vc[u] = load_stream<NT>(&c3[g]);
-        if (ACC) vo[u] = load_stream<NT>(&out[g]);
-      }
+      const uint64_t gc = g < n_groups ? g : uint64_t(n_groups) - 1u;
+      if (NIN >= 1) va[u] = load_stream<NT>(&a[gc]);
+      if (NIN >= 2) vb[u] = load_stream<NT>(&b[gc]);
+      if (NIN >= 3) vc[u] = load_stream<NT>(&c3[gc]);
+      if (ACC) vo[u] = load_stream<NT>(&out[gc]);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
