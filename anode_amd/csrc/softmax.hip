@@ -115,7 +115,21 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
     const bool mine = local < rows;  // the same for all lanes of a row's group
     const uint32_t label = (mine && nl.on()) ? nl.label(r) : 0u;
     const float dyr = (mine && nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
-    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) tile4[g] = reinterpret_cast<const f32x4 *>(xt)[g];
+    if (n4 != 0u) {
+      // the tile is at most 2048 groups, eight per thread: all requested before the first is written to LDS (a
+      // slot past the tile's end reads its last group again and is dropped)
+      f32x4 in[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t g = threadIdx.x + uint32_t(i) * kBlock;
+        in[i] = reinterpret_cast<const f32x4 *>(xt)[g < n4 ? g : n4 - 1u];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t g = threadIdx.x + uint32_t(i) * kBlock;
+        if (g < n4) tile4[g] = in[i];
+      }
+    }
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) tile[e] = xt[e];
     __syncthreads();
     float *row = tile + local * K + l;  // this lane's classes are row[0], row[G], row[2G], ...
