@@ -421,10 +421,25 @@ __global__ __launch_bounds__(kBlock) void chan_reduce_fold_kernel(uint32_t C, ui
   const double *p0 = part + size_t(c) * ppc;
   const double *p1 = p0 + size_t(C) * ppc;
   const double *p2 = p1 + size_t(C) * ppc;
-  for (uint32_t j = lane; j < ppc; j += kWave) {
-    s0 += p0[j];
-    if (Op::NACC >= 2) s1 += p1[j];
-    if (Op::NACC >= 3) s2 += p2[j];
+  // ppc <= 256 here: a lane's (up to) four partials per sum are requested together, then added in order
+  if (ppc != 0u) {
+    double v0[4], v1[4], v2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t j = lane + uint32_t(i) * kWave;
+      const uint32_t jc = j < ppc ? j : ppc - 1u;
+      v0[i] = p0[jc];
+      if (Op::NACC >= 2) v1[i] = p1[jc];
+      if (Op::NACC >= 3) v2[i] = p2[jc];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (lane + uint32_t(i) * kWave < ppc) {
+        s0 += v0[i];
+        if (Op::NACC >= 2) s1 += v1[i];
+        if (Op::NACC >= 3) s2 += v2[i];
+      }
+    }
   }
   s0 = wave_sum(s0);
   if (Op::NACC >= 2) s1 = wave_sum(s1);
