@@ -206,14 +206,26 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t
   }
   uint32_t w[4];
   wave_deal_dwords(v, lds + wave * (kWave * 4), w);
+  // the parameters of all four groups are requested before the first store (a streaming store is an ordering point
+  // for the compiler: loads written after it are issued after it); a slot past the end takes the last group's
+  uint32_t c4[4], sp4[4];
+  float a4[4], b4[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint64_t d = wave_first + uint32_t(j) * kWave + lane;
+    const uint32_t dc = (d < n_dwords) ? uint32_t(d) : (n_dwords != 0u ? n_dwords - 1u : 0u);
+    uint32_t q;
+    div_s.divmod(dc * 4u, q, sp4[j]);
+    c4[j] = q - div_c.div(q) * C;
+    a4[j] = scale[c4[j]];
+    b4[j] = shift[c4[j]];
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const uint64_t d = wave_first + uint32_t(j) * kWave + lane;
     if (d < n_dwords) {
-      uint32_t q, sp;
-      div_s.divmod(uint32_t(d) * 4u, q, sp);
-      uint32_t c = q - div_c.div(q) * C;
-      float a = scale[c], b = shift[c];
+      uint32_t sp = sp4[j], c = c4[j];
+      float a = a4[j], b = b4[j];
       f32x4 r;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
