@@ -91,7 +91,9 @@ __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uin
           const uint32_t room = S - s;  // elements of the group that still belong to channel c
           const typename Op::Param p0 = op.load(c);
           const uint32_t c1 = (c + 1 == C) ? 0 : c + 1;
-          const typename Op::Param p1 = (room < uint32_t(L)) ? op.load(c1) : p0;
+          // (fetched without a branch, from channel c again where the group does not cross: a branch round the
+          // fetch would make it wait for the loads issued before it)
+          const typename Op::Param p1 = op.load(room < uint32_t(L) ? c1 : c);
 #pragma unroll
           for (int k = 0; k < L; ++k) {
             const bool first = uint32_t(k) < room;
