@@ -299,9 +299,12 @@ def test_ref_online_average_quarter_steps(oracle):
 
 def test_arg_max_rows(oracle):
     g = np.random.default_rng(3)
-    for K, R in [(10, 32), (1000, 256), (1, 5), (64, 7), (65, 3), (5000, 2), (1001, 33), (8, 1000), (4096, 9)]:
+    for K, R in [(10, 32), (1000, 256), (1, 5), (64, 7), (65, 3), (5000, 2), (1001, 33), (8, 1000), (4096, 9),
+                 # rows that start at every distance from a 128-byte line (K = 4 * odd), few and many passes per row
+                 (12, 40), (20, 33), (100, 64), (204, 20), (1012, 17), (2044, 9), (260, 70)]:
         # a coarse grid of values: ties within a lane's group of four, across lanes and across loop passes
-        x = (g.integers(-3, 4, K * R) * 0.5).astype(F32) if K in (8, 1001, 4096) else g.standard_normal(K * R).astype(F32)
+        x = ((g.integers(-3, 4, K * R) * 0.5).astype(F32) if K in (8, 1001, 4096, 12, 100, 1012, 260)
+             else g.standard_normal(K * R).astype(F32))
         xr = x.reshape(R, K)
         if R > 3 and K > 4:
             xr[0, :] = 1.0                       # all equal: first index
