@@ -50,6 +50,8 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (10, 4000), (7, 777), (32, 600), (16, 257), (4, 1025), (5, 256), (31, 1023),
               # either side of the switch from lane groups over an LDS tile to one wave per row, 2 to 8 lanes per row
               (208, 70), (209, 70), (212, 33), (40, 1000), (96, 300), (130, 77), (200, 50),
+              # rows in registers that start at every distance from a 128-byte line (K = 4 * odd)
+              (212, 40), (1012, 19), (2044, 9), (2052, 11), (4100, 9), (8196, 3),
               # the limits of the workgroup-per-row register kernel
               (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1)]
 
