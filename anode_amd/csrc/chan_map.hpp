@@ -219,7 +219,7 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
   const bool vec = aligned16(out) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b)) &&
                    (NIN < 3 || aligned16(c));
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
-  if (vec && S == 1 && C % 4 == 0 && N >= kColSamples) {
+  if (vec && S == 1 && C % 4 == 0 && C >= 64 && N >= kColSamples) {  // (fewer channels: a wave's loads would scatter)
     const uint32_t gpp = uint32_t(uint64_t(C) * S / 4);
     const uint64_t threads = uint64_t(gpp) * ((N + kColSamples - 1) / kColSamples);  // <= len / 4
     const FastDiv div_gpp(gpp);

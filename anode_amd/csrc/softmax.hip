@@ -933,8 +933,12 @@ void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x
   pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
   if constexpr (PixVec<V>::W == 4) {
     // more classes: eight lanes per pixel group, 8, 16 or 32 sixteen-byte values per lane
-    if (C > 128) {
+    if (C > 192) {
       softmax_nd_reg_kernel<256, V, NLL, NT, 8, BWD>
+          <<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
+      return;
+    } else if (C > 128) {
+      softmax_nd_reg_kernel<192, V, NLL, NT, 8, BWD>
           <<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
       return;
     } else if (C > 64) {
@@ -989,6 +993,12 @@ void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x,
   }
 }
 
+// Which kernel takes 33 to 128 classes: one pixel per thread where 16-byte accesses are not legal, or where the
+// planes are so short that eight lanes per pixel group would read 128-byte pieces of them (P = 196, C = 64:
+// 3.7 TB/s against 2.3).  The plain and the fused entry points must agree on this: the order in which a pixel's
+// exponentials are added, hence the bits of p, depends on the kernel.
+bool nd_one_pixel_per_thread(uint32_t P, uint32_t C, bool vec) { return (!vec || P < 1024) && C > 32 && C <= 128; }
+
 void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                        CUstream_st *stream) {
   const uint32_t len = checked_len(P, C, N, symbol);
@@ -999,8 +1009,8 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
-  if (!vec && C > 32 && C <= 128) {
-    // too many classes for four pixels per thread without 16-byte accesses: one pixel per thread keeps
+  if (nd_one_pixel_per_thread(P, C, vec)) {
+    // one pixel per thread keeps
     // the row in registers and is still coalesced across the wave
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
     const uint32_t blocks = pixel_blocks(pg.total_groups);
@@ -1167,7 +1177,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll);
-             dim0 <= 32 || (vec && dim0 <= 256)) {
+             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
@@ -1196,7 +1206,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll) && aligned16(dy) && aligned16(dx);
-             dim0 <= 32 || (vec && dim0 <= 256)) {
+             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);

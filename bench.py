@@ -40,6 +40,9 @@ def parse_args():
                          "822 MB arrays under the launch-geometry and cache-policy knobs, one JSON line")
     ap.add_argument("--all-symbols", action="store_true",
                     help="instead of the benchmark: every entry point once at a bandwidth-sized shape, one JSON line")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="instead of the benchmark: batch-norm pieces over S x C, row softmax over K and channel-axis "
+                         "softmax over C x P, each on ~256 MB arrays, one JSON line (where the tilings switch)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="add one plain copy of a known size to the step (scale for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
@@ -342,6 +345,76 @@ def stream_probe(torch, gpu):
         "softmax_nd (all planes, then store)": rate(
             lambda i: gpu.call("anode_gpu_softmax_nd_packed_f32", P, Cc, Nn, *sets[i % 3]), 8 * m),
     }
+    return out
+
+
+def shape_sweep(torch, gpu):
+    """Bandwidth of the main kernel families across the shapes at which their tilings switch (algorithmic bytes /
+    time of 8 launches in rotation over cold arrays).  Every array handed to an entry point is a view of exactly the
+    element count the dims describe, checked before the call."""
+    total = 64 << 20  # elements per buffer (256 MB of f32)
+    bufs = [torch.randn(total, device="cuda") for _ in range(6)]
+    labels = torch.zeros(total, device="cuda", dtype=torch.int32)
+
+    def rate(fn, nbytes, reps=8):
+        for i in range(2):
+            fn(i)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(reps):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return round(nbytes / (a.elapsed_time(b) * 1e-3 / reps) / 1e9)
+
+    def views(n):
+        assert 0 < n <= total
+        v = [b[:n] for b in bufs]
+        assert all(t.numel() == n for t in v)
+        return v
+
+    out = {"elements_per_array_at_most": total, "unit": "GB/s of algorithmic bytes", "batch_norm": [], "row_softmax": [],
+           "nd_softmax": []}
+    for S in (1, 2, 4, 7, 16, 49, 64, 196, 256, 257, 784, 1024, 1025, 3136, 4096, 4097, 12544, 200704):
+        for C in (4, 64, 2048):
+            if S * C > total:
+                continue
+            N = min(total // (S * C), 1 << 20)
+            n = S * C * N
+            x = views(n)
+            mean, var, red = (torch.zeros(C, device="cuda"), torch.ones(C, device="cuda"), torch.empty(C, device="cuda"))
+            out["batch_norm"].append({
+                "S": S, "C": C, "N": N,
+                "batch_mean": rate(lambda i: gpu.call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, x[i % 3], red), 4 * n),
+                "batch_norm_bwd_var": rate(lambda i: gpu.call("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", S, C, N,
+                                                              x[i % 3], x[3 + i % 3], mean, var, red), 8 * n),
+                "batch_norm": rate(lambda i: gpu.call("anode_gpu_batch_norm_3d1_packed_f32", S, C, N, x[i % 3], mean, var,
+                                                      x[3 + i % 3]), 8 * n),
+                "batch_var_bwd_accumulate": rate(lambda i: gpu.call("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32",
+                                                                    S, C, N, var, x[i % 3], mean, x[3 + i % 3]), 12 * n)})
+    for K in (8, 10, 19, 32, 33, 64, 100, 128, 200, 208, 209, 256, 512, 1000, 1024, 2048, 2049, 4096, 16384, 16385, 50000):
+        R = total // K
+        n = K * R
+        x = views(n)
+        out["row_softmax"].append({
+            "K": K, "R": R,
+            "softmax_packed_block": rate(lambda i: gpu.call("anode_gpu_softmax_packed_block_f32", K, R, x[i % 3],
+                                                            x[3 + i % 3]), 8 * n)})
+    for P in (65536, 196):
+        for C in (2, 4, 19, 32, 33, 64, 100, 128, 150, 256, 300):
+            N = min(total // (P * C), 1 << 20)
+            if N < 1:
+                continue
+            n = P * C * N
+            x = views(n)
+            lab, dy = labels[:P * N], bufs[5][:P * N]
+            assert lab.numel() == P * N and dy.numel() == P * N
+            out["nd_softmax"].append({
+                "P": P, "C": C, "N": N,
+                "softmax_nd": rate(lambda i: gpu.call("anode_gpu_softmax_nd_packed_f32", P, C, N, x[i % 2], x[2 + i % 2]),
+                                   8 * n),
+                "softmax_nd_cat_nll_bwd": rate(lambda i: gpu.call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dy,
+                                                                  x[i % 2], lab, x[2 + i % 2]), 8 * n)})
     return out
 
 
@@ -667,6 +740,9 @@ def main():
     torch.cuda.set_device(0)
     if args.stream_probe:
         print(json.dumps({"stream_probe": stream_probe(torch, gpu)}), flush=True)
+        return
+    if args.shape_sweep:
+        print(json.dumps({"shape_sweep": shape_sweep(torch, gpu), "peak_gbps": HBM_PEAK_GBPS}), flush=True)
         return
     if args.all_symbols:
         print(json.dumps({"all_symbols": all_symbols(torch, gpu), "peak_gbps": HBM_PEAK_GBPS}), flush=True)
