@@ -184,7 +184,8 @@ __device__ inline float group_max(float v, int width) {
 // results meet in LDS and are added in wave order.  `lds` holds kBlock/kWave
 // values.  The result is valid in every thread.  Ends with a barrier, so `lds`
 // may be reused at once.
-template <typename T>
+// (WAVES: waves of the workgroup, kBlock / kWave unless a kernel runs larger workgroups.)
+template <typename T, int WAVES = kBlock / kWave>
 __device__ inline T block_sum(T v, T *lds) {
   v = wave_sum(v);
   const int wave = threadIdx.x / kWave;
@@ -192,12 +193,13 @@ __device__ inline T block_sum(T v, T *lds) {
   __syncthreads();
   T total = lds[0];
 #pragma unroll
-  for (int w = 1; w < kBlock / kWave; ++w) total += lds[w];
+  for (int w = 1; w < WAVES; ++w) total += lds[w];
   __syncthreads();
   return total;
 }
 
 // Workgroup maximum, same contract as block_sum.
+template <int WAVES = kBlock / kWave>
 __device__ inline float block_max(float v, float *lds) {
   v = wave_max(v);
   const int wave = threadIdx.x / kWave;
@@ -205,7 +207,7 @@ __device__ inline float block_max(float v, float *lds) {
   __syncthreads();
   float top = lds[0];
 #pragma unroll
-  for (int w = 1; w < kBlock / kWave; ++w) top = fmaxf(top, lds[w]);
+  for (int w = 1; w < WAVES; ++w) top = fmaxf(top, lds[w]);
   __syncthreads();
   return top;
 }

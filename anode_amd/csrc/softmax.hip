@@ -82,6 +82,17 @@ __device__ inline float exp_nonpos(float d) {
   const float e = __builtin_amdgcn_exp2f(t);
   return fmaf(e, r * kLn2, e);
 }
+// Marks the point from which a loaded value is known to have arrived.  The streaming stores are inline assembly,
+// which the compiler's wait-count bookkeeping does not see: where the first use of an earlier load sits in a
+// conditional block after such stores, the wait it inserts there (for "the load") also waits for every store
+// issued since, one store at a time.  Using the value once before the stores begin removes those waits.
+// (The memory clobber keeps the loads written before the mark before it, and those after it after it.)
+__device__ inline void arrived(float v) { asm volatile("" ::"v"(v) : "memory"); }
+__device__ inline void arrived(uint32_t v) { asm volatile("" ::"v"(v) : "memory"); }
+__device__ inline void arrived(f32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
+__device__ inline void arrived(u32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
+__device__ inline void issue_order_fence() { asm volatile("" ::: "memory"); }
+
 // K <= 32 * G: G = 1, 2, 4 or 8 lanes per row, up to KMAX <= 32 values per lane.  A workgroup takes 256 / G
 // consecutive rows, which are contiguous floats: they are copied to LDS as they lie in memory, 16 bytes per lane,
 // each lane group normalises its row in registers, and the tile goes back the same way, so every global access
@@ -313,16 +324,17 @@ __device__ inline void online_merge(float &m, float &s, float m2, float s2) {
   m = mm;
 }
 
-// 2048 < K <= 256 * VPT: one workgroup per row, the row in registers (VPT values per thread), so x is read once.
-// VEC as in the wave kernel.
-template <int VPT, bool VEC, int NT>
-__global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K, uint32_t R,
+// 2048 < K <= THREADS * VPT: one workgroup per row, the row in registers (VPT values per thread), so x is read once.
+// VEC as in the wave kernel.  THREADS is 256, or 1024 for rows of 16385 to 32768 classes (32 values per thread: the
+// four waves that each SIMD then holds have 128 registers each, too few for 64 values without spilling).
+template <int VPT, bool VEC, int NT, int THREADS = kBlock>
+__global__ __launch_bounds__(THREADS) void softmax_row_blockreg_kernel(uint32_t K, uint32_t R,
                                                                       const float *__restrict__ x,
                                                                       float *__restrict__ y, RowNll nl) {
   constexpr int W = VEC ? 4 : 1;
   constexpr int NG = VPT / W;
   static_assert((NG & (NG - 1)) == 0, "the wrapped lane assignment needs a power-of-two number of groups per thread");
-  __shared__ float lds[kBlock / kWave];
+  __shared__ float lds[THREADS / kWave];
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
@@ -334,8 +346,8 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
     // only, so results do not depend on where the arrays lie.
     const uint32_t a = VEC ? (uint32_t(r) * (K / 4u)) & 7u : 0u;
     auto kof = [&](int i) -> uint32_t {
-      const uint32_t slot = threadIdx.x + uint32_t(i) * kBlock;
-      return VEC ? ((slot + uint32_t(NG) * kBlock - a) & (uint32_t(NG) * kBlock - 1u)) * 4u : slot;
+      const uint32_t slot = threadIdx.x + uint32_t(i) * uint32_t(THREADS);
+      return VEC ? ((slot + uint32_t(NG) * uint32_t(THREADS) - a) & (uint32_t(NG) * uint32_t(THREADS) - 1u)) * 4u : slot;
     };
     // the row's label and upstream gradient are requested together with the row, not after the reductions
     const uint32_t label = nl.on() ? nl.label(r) : 0u;
@@ -358,7 +370,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
         m = fmaxf(m, v[i]);
       }
     }
-    m = block_max(m, lds);
+    m = block_max<THREADS / kWave>(m, lds);
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
@@ -366,7 +378,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
       v[i] = (k < K) ? exp_nonpos(v[i] - m) : 0.0f;
       s += v[i];
     }
-    s = block_sum(s, lds);
+    s = block_sum<float, THREADS / kWave>(s, lds);
     const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
@@ -394,24 +406,155 @@ __global__ __launch_bounds__(kBlock) void softmax_row_blockreg_kernel(uint32_t K
   }
 }
 
-// any K: one workgroup per row, the row streamed twice
-__global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, uint32_t R,
-                                                                   const float *__restrict__ x,
-                                                                   float *__restrict__ y, RowNll nl) {
-  __shared__ float lds_m[kBlock / kWave], lds_s[kBlock / kWave];
+// any K: workgroups of 512 threads, two to a CU, each walking rows.  A row is taken in batches of U groups of W
+// values per thread (a slot past the row's end reads the last group again and counts as -inf) and folded into a
+// running maximum and a running sum of exponentials about it; the next batch is requested before the current one
+// is folded, so the row streams in without a pause.  The first 16384 values are kept in LDS (64 KB) on the way,
+// the rest is read again by the normalising pass, which is pipelined the same way; the next row's first batch is
+// requested before the held part is written.  (One workgroup of 1024 threads per CU holding 32768 values was no
+// faster: [2047, 32772] 3.3 TB/s against 4.0, [1024, 65536] 4.6 against 4.5.  A CU that loads, reduces and stores
+// one row at a time leaves the memory system idle between the phases; two workgroups overlap them.)
+constexpr int kRowStreamThreads = 512;
+constexpr int kRowStreamHeld = 32 * kRowStreamThreads;  // values of a row that stay in LDS
+template <bool VEC, int NT>
+__global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(uint32_t K, uint32_t R,
+                                                                               const float *__restrict__ x,
+                                                                               float *__restrict__ y, RowNll nl) {
+  constexpr int THREADS = kRowStreamThreads;
+  constexpr int W = VEC ? 4 : 1;
+  constexpr int U = VEC ? 4 : 8;
+  constexpr int WAVES = THREADS / kWave;
+  constexpr uint32_t kBatch = uint32_t(THREADS) * U;  // groups per batch
+  constexpr uint32_t kHeldBatches = uint32_t(kRowStreamHeld) / (kBatch * W);
+  static_assert(kHeldBatches * kBatch * W == uint32_t(kRowStreamHeld), "whole batches are held");
+  __shared__ __align__(16) float held[kRowStreamHeld];
+  __shared__ float lds_m[WAVES], lds_s[WAVES];
+  const uint32_t groups = K / uint32_t(W);  // VEC: the host checked K % 4 == 0
+  const uint32_t batches = uint32_t((uint64_t(groups) + kBatch - 1u) / kBatch);
+  const uint32_t held_batches = batches < kHeldBatches ? batches : kHeldBatches;
+  // 64-bit group numbers: a batch's first group plus the batch can pass 2^32.  A batch past the row's end is
+  // requested like any other (it reads the row's last group) and counts for nothing.
+  auto request = [&](const float *xr, uint32_t b, float (&t)[U][W], auto last_use) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint64_t g = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x;
+      const uint32_t gc = g < groups ? uint32_t(g) : groups - 1u;
+      if (VEC) {
+        const f32x4 q = decltype(last_use)::value ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + size_t(gc) * 4u))
+                                                  : *reinterpret_cast<const f32x4 *>(xr + size_t(gc) * 4u);
+#pragma unroll
+        for (int j = 0; j < W; ++j) t[u][j] = q[j];
+      } else {
+        t[u][0] = xr[gc];
+      }
+    }
+  };
+  float ta[U][W], tb[U][W];
+  if (blockIdx.x < R) request(x + size_t(blockIdx.x) * K, 0, ta, std::false_type{});
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
     const float *xr = x + size_t(r) * K;
     float *yr = y + size_t(r) * K;
-    float m = kNegInf, s = 0.0f;
-    for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
-      const float v = xr[k];
-      if (v > m) {
-        s = (s == 0.0f) ? 1.0f : fmaf(s, exp_nonpos(m - v), 1.0f);
-        m = v;
-      } else if (!(v == kNegInf && m == kNegInf)) {
-        // a -inf seen before any larger value adds exp(-inf - max) = 0
-        s += exp_nonpos(v - m);
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
+    // the held batches: slot (b * U + u) * THREADS + threadIdx.x, written and read by the same thread
+    auto keep = [&](uint32_t b, const float (&t)[U][W]) {
+      if (b >= held_batches) return;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t slot = (b * uint32_t(U) + uint32_t(u)) * uint32_t(THREADS) + threadIdx.x;
+        if (VEC) {
+          reinterpret_cast<f32x4 *>(held)[slot] = f32x4{t[u][0], t[u][1], t[u][2], t[u][3]};
+        } else {
+          held[slot] = t[u][0];
+        }
       }
+    };
+    auto recall = [&](uint32_t b, float (&t)[U][W]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t slot = (b * uint32_t(U) + uint32_t(u)) * uint32_t(THREADS) + threadIdx.x;
+        if (VEC) {
+          const f32x4 q = reinterpret_cast<const f32x4 *>(held)[slot];
+#pragma unroll
+          for (int j = 0; j < W; ++j) t[u][j] = q[j];
+        } else {
+          t[u][0] = held[slot];
+        }
+      }
+    };
+    float m = kNegInf, s = 0.0f;
+    auto fold = [&](uint32_t b, float (&t)[U][W]) {
+      float bm = kNegInf;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool in = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x < groups;
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+          if (!in) t[u][j] = kNegInf;
+          bm = fmaxf(bm, t[u][j]);
+        }
+      }
+      float bs = 0.0f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int j = 0; j < W; ++j) bs += exp_nonpos(t[u][j] - bm);
+      }
+      if (bm == kNegInf) {
+        // a batch of -inf has seen nothing: its sum, exp(-inf - -inf) = NaN, is not a sum.  A NaN among them
+        // (which the maximum ignores) still has to reach the row's sum.
+        bool nan = false;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int j = 0; j < W; ++j) nan |= t[u][j] != t[u][j];
+        }
+        bs = nan ? __builtin_nanf("") : 0.0f;
+      }
+      online_merge(m, s, bm, bs);
+    };
+    float rs = 0.0f;
+    auto write = [&](uint32_t b, float (&t)[U][W]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {  // all of the batch is known to be there before the first store is issued
+#pragma unroll
+        for (int j = 0; j < W; ++j) arrived(t[u][j]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint64_t g = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x;
+        if (g < groups) {
+          const uint32_t k = uint32_t(g) * uint32_t(W);
+#pragma unroll
+          for (int j = 0; j < W; ++j) {
+            t[u][j] = exp_nonpos(t[u][j] - m) * rs;
+            if (nl.on()) nl.emit_nll(r, K, label, k + uint32_t(j), t[u][j]);
+          }
+          if (VEC) {
+            store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{t[u][0], t[u][1], t[u][2], t[u][3]});
+            if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
+              store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
+                               f32x4{RowNll::grad(dyr, label, k, t[u][0]), RowNll::grad(dyr, label, k + 1u, t[u][1]),
+                                     RowNll::grad(dyr, label, k + 2u, t[u][2]),
+                                     RowNll::grad(dyr, label, k + 3u, t[u][3])});
+            }
+          } else {
+            yr[k] = t[u][0];
+            if (nl.on() && nl.dx != nullptr) nl.dx[size_t(r) * K + k] = RowNll::grad(dyr, label, k, t[u][0]);
+          }
+        }
+      }
+    };
+    // ta holds the row's first batch: requested before the loop for the workgroup's first row, and by the
+    // previous row before it began to store
+#pragma unroll 1
+    for (uint32_t b = 0; b < batches; b += 2) {
+      request(xr, b + 1u, tb, std::false_type{});
+      fold(b, ta);
+      keep(b, ta);
+      request(xr, b + 2u, ta, std::false_type{});
+      fold(b + 1u, tb);
+      keep(b + 1u, tb);
     }
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
@@ -427,14 +570,25 @@ __global__ __launch_bounds__(kBlock) void softmax_row_block_kernel(uint32_t K, u
     m = lds_m[0];
     s = lds_s[0];
 #pragma unroll
-    for (int w = 1; w < kBlock / kWave; ++w) online_merge(m, s, lds_m[w], lds_s[w]);
+    for (int w = 1; w < WAVES; ++w) online_merge(m, s, lds_m[w], lds_s[w]);
     __syncthreads();
-    const float rs = 1.0f / s;
-    const uint32_t label = nl.on() ? nl.label(r) : 0u;
-    for (uint32_t k = threadIdx.x; k < K; k += kBlock) {
-      const float pr = exp_nonpos(xr[k] - m) * rs;
-      yr[k] = pr;
-      if (nl.on()) nl.emit(r, K, label, k, pr);
+    rs = 1.0f / s;
+    if (held_batches < batches) {
+      request(xr, held_batches, ta, std::true_type{});
+#pragma unroll 1
+      for (uint32_t b = held_batches; b < batches; b += 2) {
+        request(xr, b + 1u, tb, std::true_type{});
+        write(b, ta);
+        request(xr, b + 2u, ta, std::true_type{});
+        write(b + 1u, tb);
+      }
+    }
+    // the next row starts to arrive while this one's held part is written
+    if (r + gridDim.x < R) request(x + size_t(r + gridDim.x) * K, 0, ta, std::false_type{});
+#pragma unroll 1
+    for (uint32_t b = 0; b < held_batches; ++b) {
+      recall(b, tb);
+      write(b, tb);
     }
   }
 }
@@ -533,8 +687,26 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       ANODE_ROW_BLOCKREG(32);
     } else if (K <= 16384) {
       ANODE_ROW_BLOCKREG(64);
+    } else if (K <= 32768) {
+      // workgroups of 1024 threads, 32 values each
+      if (vec) {
+        with_stream_policy(nt, [&](auto policy) {
+          softmax_row_blockreg_kernel<32, true, decltype(policy)::value, 1024><<<blocks, 1024, 0, s>>>(K, R, x, y, nl);
+        });
+      } else {
+        softmax_row_blockreg_kernel<32, false, 0, 1024><<<blocks, 1024, 0, s>>>(K, R, x, y, nl);
+      }
     } else {
-      softmax_row_block_kernel<<<blocks, kBlock, 0, s>>>(K, R, x, y, nl);
+      // two workgroups per CU, which walk their rows
+      const uint32_t cus = 2u * uint32_t(device_cu_count());
+      const uint32_t walkers = R < cus ? R : cus;
+      if (vec) {
+        with_stream_policy(nt, [&](auto policy) {
+          softmax_row_stream_kernel<true, decltype(policy)::value><<<walkers, kRowStreamThreads, 0, s>>>(K, R, x, y, nl);
+        });
+      } else {
+        softmax_row_stream_kernel<false, 0><<<walkers, kRowStreamThreads, 0, s>>>(K, R, x, y, nl);
+      }
     }
 #undef ANODE_ROW_BLOCKREG
   }
@@ -616,16 +788,6 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
   p = r * uint32_t(W);
 }
 
-// Marks the point from which a loaded value is known to have arrived.  The streaming stores are inline assembly,
-// which the compiler's wait-count bookkeeping does not see: where the first use of an earlier load sits in a
-// conditional block after such stores, the wait it inserts there (for "the load") also waits for every store
-// issued since, one store at a time.  Using the value once before the stores begin removes those waits.
-// (The memory clobber keeps the loads written before the mark before it, and those after it after it.)
-__device__ inline void arrived(float v) { asm volatile("" ::"v"(v) : "memory"); }
-__device__ inline void arrived(uint32_t v) { asm volatile("" ::"v"(v) : "memory"); }
-__device__ inline void arrived(f32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
-__device__ inline void arrived(u32x4 v) { asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w) : "memory"); }
-__device__ inline void issue_order_fence() { asm volatile("" ::: "memory"); }
 
 // the value held by the lane whose number differs in the bits of `off`
 __device__ inline float lane_swap(float v, int off) { return __shfl_xor(v, off, kWave); }
@@ -790,8 +952,16 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
       for (int w = 0; w < W; ++w) {
         float mw = lane_get<V>(m, w), sw = lane_get<V>(s, w);
         const float bmw = lane_get<V>(bm, w);
-        // a block of -inf planes has seen nothing: its sum, exp(-inf - -inf) = NaN, is not a sum
-        online_merge(mw, sw, bmw, bmw == kNegInf ? 0.0f : lane_get<V>(bs, w));
+        float bsw = lane_get<V>(bs, w);
+        if (bmw == kNegInf) {
+          // a block of -inf planes has seen nothing: its sum, exp(-inf - -inf) = NaN, is not a sum.  A NaN among
+          // them (which the maximum ignores) still has to reach the pixel's sum.
+          bool nan = false;
+#pragma unroll
+          for (int u = 0; u < U; ++u) nan |= lane_get<V>(v[u], w) != lane_get<V>(v[u], w);
+          bsw = nan ? __builtin_nanf("") : 0.0f;
+        }
+        online_merge(mw, sw, bmw, bsw);
         lane_set<V>(m, w, mw);
         lane_set<V>(s, w, sw);
       }

@@ -53,7 +53,10 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               # rows in registers that start at every distance from a 128-byte line (K = 4 * odd)
               (212, 40), (1012, 19), (2044, 9), (2052, 11), (4100, 9), (8196, 3),
               # the limits of the workgroup-per-row register kernel
-              (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1)]
+              (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1),
+              # workgroups of 1024 threads: rows in registers up to 32768 classes, streamed twice beyond
+              (16388, 3), (20000, 3), (32764, 2), (32768, 2), (32769, 1), (32772, 3), (50257, 2), (65536, 2),
+              (65540, 1), (100003, 1), (262148, 2)]
 
 
 @pytest.mark.parametrize("K,R", ROW_SHAPES)
@@ -96,6 +99,41 @@ def test_softmax_rows_special_values(oracle):
     y2 = empty(3 * K2)
     call("anode_gpu_softmax_packed_deterministic_f32", K2, 3, dev(x2), y2)
     assert_close(host(y2), oracle.softmax(K2, 3, x2.ravel(), f64=True), "block kernel special values", abs_floor=1e-30)
+
+
+@pytest.mark.parametrize("K", [20000, 40004, 70001, 140000])
+def test_softmax_long_rows_special_values(oracle, K):
+    # rows of 1024-thread workgroups (in registers) and rows that are streamed in batches with a running maximum:
+    # batches of nothing but -inf before, between and after the finite values, the maximum in the first or in the
+    # last batch, a NaN in the part that is read twice, a row of nothing but -inf
+    R = 9
+    print(f"case long rows K={K}", flush=True)
+    x = np.full((R, K), -np.inf, F32)
+    x[0, K - 3] = 2.0
+    x[1, :] = 0.5
+    x[1, :K // 2] = -np.inf
+    x[2, :] = np.linspace(-50, 50, K)
+    x[3, :] = np.linspace(50, -50, K)
+    x[4, :] = 1.0
+    x[4, K - 1] = np.nan
+    x[5, 5] = 3.0
+    x[5, K // 2] = 3.0
+    x[6, :] = 88.0
+    x[7, :] = np.random.default_rng(K).standard_normal(K).astype(F32)
+    x[7, K // 3] = 1e30
+    # row 8 stays -inf throughout: NaN, as exp(-inf - -inf) is
+    for offset in (0, 1):
+        y = empty(K * R, offset=offset)
+        call("anode_gpu_softmax_packed_deterministic_f32", K, R, dev(x, offset), y)
+        p = host(y).reshape(R, K)
+        want = oracle.softmax(K, R, x.ravel(), f64=True).reshape(R, K)
+        assert_close(p, want, f"long rows K={K}", abs_floor=1e-30)
+        assert p[0, K - 3] == 1.0 and np.count_nonzero(p[0]) == 1
+        assert np.all(p[1, :K // 2] == 0)
+        assert np.all(np.isnan(p[4])) and np.all(np.isnan(p[8]))
+        assert p[5, 5] == 0.5 and p[5, K // 2] == 0.5
+        assert p[7, K // 3] == 1.0
+        assert not np.any(np.isnan(p[[0, 1, 2, 3, 5, 6, 7]]))
 
 
 @pytest.mark.parametrize("K,R", [(10, 32), (1000, 256), (7, 5), (1, 9), (300, 11)])
@@ -195,6 +233,9 @@ def test_softmax_nd_special_values(oracle, C):
     x[0, :, 4] = np.linspace(-60, 8, C)
     x[1, :, 5] = np.linspace(-20, 20, C)
     x[1, :, 6] = -np.inf          # nothing but -inf: NaN, as exp(-inf - -inf) is
+    x[1, :, 7] = -np.inf          # a NaN whose neighbours are all -inf still poisons its pixel
+    x[1, C - 1, 7] = np.nan
+    x[1, 0, 7] = 1.0
     for offset in (0, 1):
         y = empty(x.size, offset=offset)
         call("anode_gpu_softmax_nd_packed_f32", P, C, N, dev(x, offset), y)
