@@ -213,7 +213,7 @@ __global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t n_dwords, 
   const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // the wave's first dword
   u32x4 v = {0u, 0u, 0u, 0u};
   if (g16 * 4u + 3u < n_dwords) {
-    v = load_stream<NT>(&x16[g16]);
+    v = load_stream<kNtLoad>(&x16[g16]);  // the codes are read once, whatever the size
   } else if (g16 * 4u < n_dwords) {  // the last, partial group of the array: dword by dword
     const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
     for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = x4[g16 * 4u + k];

@@ -919,30 +919,44 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
 // any C: one pass over the classes that keeps a running maximum and a running sum of exponentials, eight planes
 // requested at a time, then a normalising pass (x is read twice; the reference reads it three times).  A block of
 // planes is folded into (its maximum, the sum of its exponentials about that maximum) and merged with the running
-// pair by online_merge(), which also keeps -inf planes from turning into NaN.
-template <typename V>
+// pair by online_merge(), which also keeps -inf planes from turning into NaN.  SPLIT lanes (1 or 8) share a group
+// of W pixels, lane h taking the classes h, h + SPLIT, ...: with few pixels and many classes one lane per group
+// leaves most of the GPU without work ([65536, 300, 3]: 192 workgroups).
+template <typename V, int SPLIT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                    float *__restrict__ y) {
   constexpr int W = PixVec<V>::W;
   constexpr int U = 8;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
+  const uint64_t total = uint64_t(pg.total_groups) * SPLIT;
+  for (uint64_t t = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
+    // the lanes of a group are neighbours, so they always run, and leave the loop, together
+    const uint32_t g = uint32_t(t / SPLIT), h = uint32_t(t % SPLIT);
     uint32_t p, n;
-    pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
+    pixel_decode(pg, g, W, p, n);  // g < total_groups, which fits 32 bits
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
     V m = PixVec<V>::splat(kNegInf);
     V s = PixVec<V>::splat(0.0f);
-    for (uint32_t k0 = 0; k0 < pg.C; k0 += U) {
+    auto merge = [&](V bm, V bs) {
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        float mw = lane_get<V>(m, w), sw = lane_get<V>(s, w);
+        online_merge(mw, sw, lane_get<V>(bm, w), lane_get<V>(bs, w));
+        lane_set<V>(m, w, mw);
+        lane_set<V>(s, w, sw);
+      }
+    };
+    for (uint32_t k0 = h; k0 < pg.C; k0 += uint32_t(U * SPLIT)) {
       V v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {  // a slot past the last class reads the last class again and is set to -inf
-        const uint32_t k = k0 + uint32_t(u);
+        const uint32_t k = k0 + uint32_t(u * SPLIT);
         v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
       }
       V bm = PixVec<V>::splat(kNegInf);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (k0 + uint32_t(u) >= pg.C) v[u] = PixVec<V>::splat(kNegInf);
+        if (k0 + uint32_t(u * SPLIT) >= pg.C) v[u] = PixVec<V>::splat(kNegInf);
         bm = vmax(bm, v[u]);
       }
       V bs = PixVec<V>::splat(0.0f);
@@ -950,33 +964,35 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
       for (int u = 0; u < U; ++u) bs += vexp(v[u] - bm);
 #pragma unroll
       for (int w = 0; w < W; ++w) {
-        float mw = lane_get<V>(m, w), sw = lane_get<V>(s, w);
-        const float bmw = lane_get<V>(bm, w);
-        float bsw = lane_get<V>(bs, w);
-        if (bmw == kNegInf) {
+        if (lane_get<V>(bm, w) == kNegInf) {
           // a block of -inf planes has seen nothing: its sum, exp(-inf - -inf) = NaN, is not a sum.  A NaN among
           // them (which the maximum ignores) still has to reach the pixel's sum.
           bool nan = false;
 #pragma unroll
           for (int u = 0; u < U; ++u) nan |= lane_get<V>(v[u], w) != lane_get<V>(v[u], w);
-          bsw = nan ? __builtin_nanf("") : 0.0f;
+          lane_set<V>(bs, w, nan ? __builtin_nanf("") : 0.0f);
         }
-        online_merge(mw, sw, bmw, bsw);
-        lane_set<V>(m, w, mw);
-        lane_set<V>(s, w, sw);
       }
+      merge(bm, bs);
+    }
+    // the lanes of the group exchange their pairs: after the last step every lane holds the same maximum, and
+    // the same sum (a + b == b + a at every step)
+#pragma unroll
+    for (int off = 1; off < SPLIT; off <<= 1) {
+      const V m2 = lane_swap(m, off), s2 = lane_swap(s, off);
+      merge(m2, s2);
     }
     const V inv = vrcp(s);
-    for (uint32_t k0 = 0; k0 < pg.C; k0 += U) {
+    for (uint32_t k0 = h; k0 < pg.C; k0 += uint32_t(U * SPLIT)) {
       V v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t k = k0 + uint32_t(u);
+        const uint32_t k = k0 + uint32_t(u * SPLIT);
         v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t k = k0 + uint32_t(u);
+        const uint32_t k = k0 + uint32_t(u * SPLIT);
         if (k < pg.C) *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = vexp(v[u] - m) * inv;
       }
     }
@@ -1020,9 +1036,12 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
                                                                         const float *__restrict__ dy,
                                                                         const float *__restrict__ prob,
                                                                         const uint32_t *__restrict__ cat,
-                                                                        float *dx) {
+                                                                        float *dx, uint32_t chunk) {
   constexpr int W = PixVec<V>::W;
   typedef typename PixVec<V>::U U;
+  // blockIdx.y picks a run of `chunk` classes (a multiple of the four that are walked together)
+  const uint32_t k_first = blockIdx.y * chunk;
+  const uint32_t k_end = k_first + chunk < pg.C ? k_first + chunk : pg.C;
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
   for (uint64_t g = uint64_t(pg.xcd ? xcd_contiguous(blockIdx.x, gridDim.x) : blockIdx.x) * kBlock + threadIdx.x; g < pg.total_groups; g += stride) {
     uint32_t p, n;
@@ -1044,7 +1063,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
     auto request = [&](uint32_t k0) {
 #pragma unroll
       for (int u = 0; u < B; ++u) {
-        const uint32_t k = k0 + uint32_t(u) < pg.C ? k0 + uint32_t(u) : pg.C - 1u;
+        const uint32_t k = k0 + uint32_t(u) < k_end ? k0 + uint32_t(u) : k_end - 1u;
         const size_t off = base + size_t(pg.P) * k;
         pr[u] = load_stream<NT>(reinterpret_cast<const V *>(prob + off));
         if (ACC) old[u] = load_stream<NT>(reinterpret_cast<const V *>(dx + off));
@@ -1054,7 +1073,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
 #pragma unroll
       for (int u = 0; u < B; ++u) {
         const uint32_t k = k0 + uint32_t(u);
-        if (k < pg.C) {
+        if (k < k_end) {
           V r;
 #pragma unroll
           for (int w = 0; w < W; ++w) {
@@ -1065,11 +1084,11 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
         }
       }
     };
-    request(0);
+    request(k_first);
     arrived(d);  // dy and the labels were requested first: known to be there before the first store is issued
     arrived(lab);
-    write(0);
-    for (uint32_t k0 = uint32_t(B); k0 < pg.C; k0 += uint32_t(B)) {
+    write(k_first);
+    for (uint32_t k0 = k_first + uint32_t(B); k0 < k_end; k0 += uint32_t(B)) {
       request(k0);
       write(k0);
     }
@@ -1159,7 +1178,12 @@ void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x,
     launch_softmax_nd_reg<V, false>(P, C, N, x, y, nullptr, nullptr, s);
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
-    softmax_nd_stream_kernel<V><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, x, y);
+    // eight lanes per pixel group unless one lane per group already fills the GPU
+    if (uint64_t(pg.total_groups) < uint64_t(device_cu_count()) * 2048u) {
+      softmax_nd_stream_kernel<V, 8><<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y);
+    } else {
+      softmax_nd_stream_kernel<V, 1><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, x, y);
+    }
   }
 }
 
@@ -1226,6 +1250,20 @@ void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint3
   note_launch(symbol);
 }
 
+// The backward pass is a map, so with few pixels and many classes the classes are shared out as well: runs of
+// `chunk` classes (a multiple of 16: a thread reads its pixels' dy and labels once per run) over blockIdx.y, as
+// many as it takes to give the GPU eight workgroups per CU ([65536, 256, 4]: 256 workgroups of pixel groups).
+dim3 nd_bwd_grid(uint32_t total_groups, uint32_t C, uint32_t &chunk) {
+  const uint32_t bx = pixel_blocks(total_groups);
+  const uint32_t want = uint32_t(device_cu_count()) * 8u;
+  uint32_t runs = bx >= want ? 1u : (want + bx - 1u) / bx;
+  const uint32_t most = (C + 15u) / 16u;
+  if (runs > most) runs = most;
+  chunk = ((C + runs - 1u) / runs + 15u) / 16u * 16u;
+  runs = (C + chunk - 1u) / chunk;
+  return dim3(bx, runs, 1);
+}
+
 template <bool ACC>
 void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *dy,
                                    const float *prob, const uint32_t *cat, float *dx, CUstream_st *stream,
@@ -1238,16 +1276,19 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
+  uint32_t chunk = C;
   if (vec) {
     PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
     pg.xcd = (tuning().nd_xcd_mask & 2) ? 1u : 0u;
+    const dim3 grid = nd_bwd_grid(pg.total_groups, C, chunk);
     with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
       softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, decltype(policy)::value>
-          <<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+          <<<grid, kBlock, 0, s>>>(pg, dy, prob, cat, dx, chunk);
     });
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, 1, ignore);
-    softmax_nd_cat_nll_bwd_kernel<float, ACC, 0><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, dy, prob, cat, dx);
+    const dim3 grid = nd_bwd_grid(pg.total_groups, C, chunk);
+    softmax_nd_cat_nll_bwd_kernel<float, ACC, 0><<<grid, kBlock, 0, s>>>(pg, dy, prob, cat, dx, chunk);
   }
   note_launch(symbol);
 }
