@@ -231,7 +231,7 @@ uint32_t pick_row_rotation(uint32_t K, uint32_t log2g) {
   return best;
 }
 
-// 208 < K <= 64 * VPL: one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
+// Up to 64 * VPL columns (from 225 on, see the dispatch): one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
 // of 4, aligned arrays) and a lane owns groups of four consecutive classes; otherwise lane l owns k = l, l+64, ...
 template <int VPL, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
@@ -603,10 +603,12 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   const uint32_t max_blocks = 1u << 24;
   constexpr uint32_t kWavesPerBlock = kBlock / kWave;
   const int nt = stream_policy(size_t(K) * R * sizeof(float), tuning().nontemporal);  // logits in, probabilities out: both streamed
-  if (K <= 208) {
+  if (K <= 224 || (K <= 256 && K % 16u != 0)) {
     // 1, 2, 4 or 8 lanes per row, at most 32 values per lane; the tile of 256 / G rows is at most 32 KiB.
-    // (From 209 columns on the wave-per-row kernel below keeps enough of its 64 lanes busy to be faster:
-    // 6.1 TB/s against 4.5 at 256 columns, 4.3 against 4.7 at 200.)
+    // The kernel is built for 4, 8, 16, 20, 24, 28 or 32 values per lane: the registers of a lane's array are what
+    // limits the waves per SIMD (K = 33 with room for 32 values per lane: 3.7 TB/s, for 20: 5.6).
+    // (Rows of 240 and 256 columns go to the wave-per-row kernel below, whose lanes then all take whole 64-byte
+    // pieces: 5.9 and 6.1 TB/s against 5.4 and 5.5 here; at 232 columns it runs at 4.9 against 5.4 here.)
     uint32_t log2g = 0;
     while ((32u << log2g) < K) ++log2g;
     const uint32_t G = 1u << log2g, KJ = (K + G - 1) / G;
@@ -634,14 +636,25 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
           launch(std::integral_constant<int, 32>{}, lg);
         }
       };
+      auto with_kmax_wide = [&](auto lg) {  // several lanes per row: 17 to 32 values per lane
+        if (KJ <= 20) {
+          launch(std::integral_constant<int, 20>{}, lg);
+        } else if (KJ <= 24) {
+          launch(std::integral_constant<int, 24>{}, lg);
+        } else if (KJ <= 28) {
+          launch(std::integral_constant<int, 28>{}, lg);
+        } else {
+          launch(std::integral_constant<int, 32>{}, lg);
+        }
+      };
       if (log2g == 0) {
         with_kmax(std::integral_constant<int, 0>{});
       } else if (log2g == 1) {
-        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 1>{});  // 32 < K <= 64: 17 to 32 values
+        with_kmax_wide(std::integral_constant<int, 1>{});
       } else if (log2g == 2) {
-        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 2>{});
+        with_kmax_wide(std::integral_constant<int, 2>{});
       } else {
-        launch(std::integral_constant<int, 32>{}, std::integral_constant<int, 3>{});
+        with_kmax_wide(std::integral_constant<int, 3>{});
       }
     });
   } else if (K <= 2048) {

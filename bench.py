@@ -392,7 +392,7 @@ def shape_sweep(torch, gpu):
                                                       x[3 + i % 3]), 8 * n),
                 "batch_var_bwd_accumulate": rate(lambda i: gpu.call("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32",
                                                                     S, C, N, var, x[i % 3], mean, x[3 + i % 3]), 12 * n)})
-    for K in (8, 10, 19, 32, 33, 64, 100, 128, 200, 208, 209, 256, 512, 1000, 1024, 2048, 2049, 4096, 16384, 16385,
+    for K in (8, 10, 19, 32, 33, 64, 100, 128, 200, 224, 232, 240, 256, 512, 1000, 1024, 2048, 2049, 4096, 16384, 16385,
               32768, 32772, 50000, 50257, 65536, 262144):
         R = total // K
         n = K * R

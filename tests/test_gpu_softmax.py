@@ -50,6 +50,10 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (10, 4000), (7, 777), (32, 600), (16, 257), (4, 1025), (5, 256), (31, 1023),
               # either side of the switch from lane groups over an LDS tile to one wave per row, 2 to 8 lanes per row
               (208, 70), (209, 70), (212, 33), (40, 1000), (96, 300), (130, 77), (200, 50),
+              (224, 33), (225, 33), (232, 17), (239, 40), (240, 9), (241, 9), (250, 21), (255, 19), (256, 33), (257, 5),
+              # every count of values per lane the tile kernel is built for, one to eight lanes per row
+              (20, 300), (24, 100), (28, 70), (36, 300), (47, 70), (52, 90), (75, 50), (92, 64), (108, 40), (150, 33),
+              (180, 41), (215, 37),
               # rows in registers that start at every distance from a 128-byte line (K = 4 * odd)
               (212, 40), (1012, 19), (2044, 9), (2052, 11), (4100, 9), (8196, 3),
               # the limits of the workgroup-per-row register kernel
