@@ -60,7 +60,10 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1),
               # workgroups of 1024 threads: rows in registers up to 32768 classes, streamed twice beyond
               (16388, 3), (20000, 3), (32764, 2), (32768, 2), (32769, 1), (32772, 3), (50257, 2), (65536, 2),
-              (65540, 1), (100003, 1), (262148, 2)]
+              (65540, 1), (100003, 1), (262148, 2),
+              # more long rows than the streaming kernel has workgroups: each walks several rows, the next row's
+              # first batch requested while the current row is written
+              (32772, 1100), (33001, 1030)]
 
 
 @pytest.mark.parametrize("K,R", ROW_SHAPES)
