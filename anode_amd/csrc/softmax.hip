@@ -933,8 +933,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
 // requested at a time, then a normalising pass (x is read twice; the reference reads it three times).  A block of
 // planes is folded into (its maximum, the sum of its exponentials about that maximum) and merged with the running
 // pair by online_merge(), which also keeps -inf planes from turning into NaN.  SPLIT lanes (1 or 8) share a group
-// of W pixels, lane h taking the classes h, h + SPLIT, ...: with few pixels and many classes one lane per group
-// leaves most of the GPU without work ([65536, 300, 3]: 192 workgroups).
+// of W pixels, lane h taking the classes h, h + SPLIT, ...: one lane per group of four pixels leaves most of the
+// GPU without work when there are few pixels and many classes ([65536, 300, 3]: 192 workgroups).
 template <typename V, int SPLIT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                    float *__restrict__ y) {
@@ -1191,8 +1191,10 @@ void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x,
     launch_softmax_nd_reg<V, false>(P, C, N, x, y, nullptr, nullptr, s);
   } else {
     const PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W);
-    // eight lanes per pixel group unless one lane per group already fills the GPU
-    if (uint64_t(pg.total_groups) < uint64_t(device_cu_count()) * 2048u) {
+    // Groups of four pixels: eight lanes per group, which is faster however many groups there are ([65536, 300, 3]
+    // 3.3 TB/s against 2.3, [4096, 1000, 16] 3.3 against 0.9).  Single pixels: one lane each, so that a wave's
+    // load still covers 256 contiguous bytes ([65535, 300, 3] 2.9 TB/s against 1.8 with eight lanes per pixel).
+    if (PixVec<V>::W == 4) {
       softmax_nd_stream_kernel<V, 8><<<stream_grid(uint64_t(pg.total_groups) * 8, 1), kBlock, 0, s>>>(pg, x, y);
     } else {
       softmax_nd_stream_kernel<V, 1><<<pixel_blocks(pg.total_groups), kBlock, 0, s>>>(pg, x, y);
