@@ -1202,6 +1202,144 @@ void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x,
   }
 }
 
+// Short planes that are not whole 64-byte pieces (P < 1024, P % 16 != 0), up to 64 classes, samples of at most
+// 32 KB: a workgroup copies SB whole samples (SB * P * C contiguous floats, 16 KB where several fit) to LDS as they
+// lie in memory, 16 bytes per lane, one thread per pixel walks its classes there (consecutive threads take
+// consecutive pixels: consecutive banks), and the tile goes back the same way; with a gradient to write, the tile
+// is turned into dy * (p - onehot) in place and goes out once more.  Every global access is full-width whatever P
+// is, where the register kernels read a [196, C] sample plane by plane in 784-byte pieces: [196, 19] 4.2 -> 5.0
+// TB/s, [196, 32] 3.5 -> 5.6, [49, 19] 4.4 -> 5.0, [4, 19] 1.4 -> 5.4.  (Planes of whole 64-byte pieces are as
+// fast or faster through the register kernels: [16, 10] 6.0 TB/s against 5.5, [784, 4] 6.1 against 5.7; so are
+// pixels of more than 64 classes, which leave most of a tile's threads idle: [4, 512] 3.0 against 1.0.)
+// A pixel's sum starts at class (sample's place in the tile) mod C and wraps round, so that samples whose size is
+// a multiple of the 32 banks do not all meet in the same banks; the order of a pixel's sum therefore depends on
+// the shape and on the sample number, and on nothing else.  All entry points (plain, with the label gather, with
+// the backward pass) run this kernel for these shapes, whatever the alignment of their arrays: their
+// probabilities agree to the bit.
+constexpr uint32_t kNdTileFloats = 4096;      // samples are gathered into tiles of 16 KB
+constexpr uint32_t kNdTileMaxSample = 8192;   // a larger sample has a tile to itself, up to 32 KB
+bool nd_tile_fits(uint32_t P, uint32_t C) {
+  return P > 1 && P < 1024 && P % 16u != 0 && C <= 64 && uint64_t(P) * C <= kNdTileMaxSample;
+}
+
+template <bool NLL, bool BWD, int NT>
+__global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uint32_t C, uint32_t N, uint32_t SB,
+                                                                 FastDiv div_p, FastDiv div_c, int vec, uint32_t ignore,
+                                                                 const float *__restrict__ x, float *__restrict__ y,
+                                                                 const uint32_t *__restrict__ cat,
+                                                                 float *__restrict__ nll,
+                                                                 const float *__restrict__ dy,
+                                                                 float *__restrict__ dx) {
+  extern __shared__ __align__(16) float tile[];  // SB * P * C floats, at most kNdTileMaxSample
+  f32x4 *tile4 = reinterpret_cast<f32x4 *>(tile);
+  const uint32_t slab = P * C;
+  for (uint64_t n0 = uint64_t(blockIdx.x) * SB; n0 < N; n0 += uint64_t(gridDim.x) * SB) {
+    const uint32_t samples = (N - n0 < uint64_t(SB)) ? uint32_t(N - n0) : SB;
+    const uint32_t n = samples * slab;
+    const uint32_t n4 = vec ? n / 4u : 0u;  // (the host checked that every tile starts on a 16-byte boundary)
+    const float *xt = x + n0 * slab;
+    float *yt = y + n0 * slab;
+    // eight groups per thread are requested before the first is written to LDS (a slot past the tile's end reads
+    // its last group again and is dropped)
+    for (uint32_t g0 = 0; g0 < n4; g0 += 8u * kBlock) {
+      f32x4 in[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t g = g0 + threadIdx.x + uint32_t(i) * kBlock;
+        in[i] = load_stream<NT>(reinterpret_cast<const f32x4 *>(xt) + (g < n4 ? g : n4 - 1u));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t g = g0 + threadIdx.x + uint32_t(i) * kBlock;
+        if (g < n4) tile4[g] = in[i];
+      }
+    }
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) tile[e] = xt[e];
+    __syncthreads();
+    const uint32_t pixels = samples * P;
+    const size_t pix0 = size_t(n0) * P;
+    for (uint32_t q = threadIdx.x; q < pixels; q += kBlock) {
+      uint32_t sb, pp;
+      div_p.divmod(q, sb, pp);
+      // the label is requested before the walk, so that it is there after it
+      uint32_t label = 0u;
+      if (NLL) label = cat[pix0 + q];
+      float *col = tile + sb * slab + pp;  // class k of this pixel is col[k * P]
+      const uint32_t first = sb - div_c.div(sb) * C;
+      float m = kNegInf;
+#pragma unroll 4
+      for (uint32_t k = 0; k < C; ++k) m = fmaxf(m, col[k * P]);
+      float sum = 0.0f;  // classes first .. C - 1, then 0 .. first - 1
+#pragma unroll 4
+      for (uint32_t k = first; k < C; ++k) {
+        const float e = exp_nonpos(col[k * P] - m);
+        col[k * P] = e;
+        sum += e;
+      }
+#pragma unroll 4
+      for (uint32_t k = 0; k < first; ++k) {
+        const float e = exp_nonpos(col[k * P] - m);
+        col[k * P] = e;
+        sum += e;
+      }
+      const float inv = 1.0f / sum;  // one correctly rounded reciprocal per pixel
+#pragma unroll 4
+      for (uint32_t k = 0; k < C; ++k) col[k * P] *= inv;
+      if (NLL) {
+        // -log of the stored probability of the label; NaN (0 with `ignore`) when the label is out of range
+        nll[pix0 + q] = label < C ? -logf(col[label * P]) : (ignore ? 0.0f : __builtin_nanf(""));
+      }
+    }
+    __syncthreads();
+    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, tile4[g]);
+    for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) yt[e] = tile[e];
+    __syncthreads();  // the tile is overwritten below, or by the next pass
+    if (BWD) {
+      for (uint32_t q = threadIdx.x; q < pixels; q += kBlock) {
+        uint32_t sb, pp;
+        div_p.divmod(q, sb, pp);
+        const uint32_t label = cat[pix0 + q];
+        float d = dy[pix0 + q];
+        if (ignore && label >= C) d = 0.0f;
+        float *col = tile + sb * slab + pp;
+#pragma unroll 4
+        for (uint32_t k = 0; k < C; ++k) col[k * P] = d * (col[k * P] - float(label == k));
+      }
+      __syncthreads();
+      float *dt = dx + n0 * slab;
+      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, tile4[g]);
+      for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) dt[e] = tile[e];
+      __syncthreads();
+    }
+  }
+}
+
+template <bool NLL, bool BWD>
+void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, float *y, const uint32_t *cat,
+                            float *nll, const float *dy, float *dx, bool ignore, hipStream_t s) {
+  const uint32_t slab = P * C;
+  // as many samples as fit, but no more than leaves every CU two workgroups; from four on a multiple of four,
+  // so that every tile starts on a 16-byte boundary
+  uint32_t SB = kNdTileFloats / slab;
+  const uint32_t spread = (N + 2u * uint32_t(device_cu_count()) - 1u) / (2u * uint32_t(device_cu_count()));
+  if (SB > spread) SB = spread;
+  if (SB >= 4u) SB &= ~3u;
+  if (SB == 0u) SB = 1u;
+  uint32_t blocks = (N + SB - 1u) / SB;
+  const uint32_t max_blocks = 1u << 24;
+  if (blocks > max_blocks) blocks = max_blocks;
+  const bool starts_aligned = (uint64_t(SB) * slab) % 4u == 0 || N <= SB;
+  const int vec = (starts_aligned && aligned16(x) && aligned16(y) && (!BWD || aligned16(dx))) ? 1 : 0;
+  const size_t lds_bytes = size_t(SB) * slab * sizeof(float);
+  const FastDiv div_p(P), div_c(C);
+  // logits in, probabilities (and the gradient) out: all streamed
+  const int nt = stream_policy(size_t(slab) * N * sizeof(float), tuning().nontemporal);
+  with_stream_policy(nt, [&](auto policy) {
+    softmax_nd_tile_kernel<NLL, BWD, decltype(policy)::value>
+        <<<blocks, kBlock, lds_bytes, s>>>(P, C, N, SB, div_p, div_c, vec, ignore ? 1u : 0u, x, y, cat, nll, dy, dx);
+  });
+}
+
 // Which kernel takes 33 to 128 classes: one pixel per thread where 16-byte accesses are not legal, or where the
 // planes are so short that eight lanes per pixel group would read 128-byte pieces of them (P = 196, C = 64:
 // 3.7 TB/s against 2.3).  The plain and the fused entry points must agree on this: the order in which a pixel's
@@ -1218,7 +1356,9 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
-  if (nd_one_pixel_per_thread(P, C, vec)) {
+  if (nd_tile_fits(P, C)) {
+    launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+  } else if (nd_one_pixel_per_thread(P, C, vec)) {
     // one pixel per thread keeps
     // the row in registers and is still coalesced across the wave
     const PixelGrid pg = make_pixel_grid(P, C, N, 1);
@@ -1265,6 +1405,41 @@ void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint3
   note_launch(symbol);
 }
 
+// The same map for planes shorter than 1024 pixels, walked as the flat array it is: a thread takes one 16-byte group
+// of dx (four consecutive pixels of one class), so a wave's accesses are 1 KiB contiguous however short the planes
+// are, and fetches its pixels' dy and labels from the caches (every class of a sample asks for the same ones).
+// [196, 19, 18020]: 3.6 -> 5.5 TB/s.  The arithmetic is that of the kernel above.
+template <bool ACC, int NT>
+__global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_kernel(uint32_t P, uint32_t C, uint32_t total_groups,
+                                                                             FastDiv div_gpp, FastDiv div_c, uint32_t ignore,
+                                                                             const float *__restrict__ dy,
+                                                                             const float *__restrict__ prob,
+                                                                             const uint32_t *__restrict__ cat,
+                                                                             float *dx) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g64 = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g64 < total_groups; g64 += stride) {
+    const uint32_t g = uint32_t(g64);
+    uint32_t plane, r;  // plane = n * C + k, r = the group's place in the plane
+    div_gpp.divmod(g, plane, r);
+    const uint32_t n = div_c.div(plane);
+    const uint32_t k = plane - n * C;
+    const size_t pix = size_t(n) * P + size_t(r) * 4u;
+    f32x4 d = *reinterpret_cast<const f32x4 *>(dy + pix);
+    const u32x4 lab = *reinterpret_cast<const u32x4 *>(cat + pix);
+    const f32x4 pr = load_stream<NT>(reinterpret_cast<const f32x4 *>(prob) + g);
+    f32x4 old = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (ACC) old = load_stream<NT>(reinterpret_cast<const f32x4 *>(dx) + g);
+    f32x4 out;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (ignore && lab[w] >= C) d[w] = 0.0f;
+      const float t = pr[w] - float(lab[w] == k);
+      out[w] = ACC ? fmaf(d[w], t, old[w]) : d[w] * t;
+    }
+    store_stream<NT>(reinterpret_cast<f32x4 *>(dx) + g, out);
+  }
+}
+
 // The backward pass is a map, so with few pixels and many classes the classes are shared out as well: runs of
 // `chunk` classes (a multiple of 16: a thread reads its pixels' dy and labels once per run) over blockIdx.y, as
 // many as it takes to give the GPU eight workgroups per CU ([65536, 256, 4]: 256 workgroups of pixel groups).
@@ -1292,7 +1467,15 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   uint32_t chunk = C;
-  if (vec) {
+  if (vec && P < 1024) {
+    const uint32_t total_groups = len / 4u;
+    const FastDiv div_gpp(P / 4u), div_c(C);
+    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
+      softmax_nd_cat_nll_bwd_flat_kernel<ACC, decltype(policy)::value>
+          <<<stream_grid(total_groups, 1), kBlock, 0, s>>>(P, C, total_groups, div_gpp, div_c, ignore ? 1u : 0u, dy, prob,
+                                                          cat, dx);
+    });
+  } else if (vec) {
     PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
     pg.xcd = (tuning().nd_xcd_mask & 2) ? 1u : 0u;
     const dim3 grid = nd_bwd_grid(pg.total_groups, C, chunk);
@@ -1401,6 +1584,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
+  } else if (nd_tile_fits(prefix_dim, dim0)) {
+    launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
+                                        as_stream(stream));
+    note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll);
              dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
@@ -1430,6 +1617,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
+  } else if (nd_tile_fits(prefix_dim, dim0)) {
+    launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
+                                       as_stream(stream));
+    note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll) && aligned16(dy) && aligned16(dx);
              dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {

@@ -186,7 +186,15 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
 
 @pytest.mark.parametrize("P,C,N", [(64, 19, 2), (2048, 19, 2), (5, 3, 4), (1, 10, 6), (16, 32, 2), (8, 40, 3), (100, 1, 3),
                                    (1300, 19, 3), (516, 24, 2), (1028, 2, 3), (12, 7, 5),
-                                   (20, 48, 3), (24, 129, 2), (16, 200, 2), (8, 256, 3), (8, 300, 2), (520, 40, 2)])
+                                   (20, 48, 3), (24, 129, 2), (16, 200, 2), (8, 256, 3), (8, 300, 2), (520, 40, 2),
+                                   # planes of 1024 pixels and more: the register and streaming kernels
+                                   (1028, 8, 2), (1024, 32, 2), (1028, 48, 2), (1032, 65, 2), (1028, 129, 1),
+                                   (1024, 192, 1), (1024, 256, 2), (1028, 300, 1), (1025, 19, 2), (1025, 40, 2),
+                                   (1025, 130, 1),
+                                   # short planes through the LDS tile, and its neighbours
+                                   (196, 32, 9), (196, 41, 5), (196, 42, 3), (1023, 8, 3), (127, 64, 3), (127, 65, 3),
+                                   (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 2, 9000), (512, 32, 3), (196, 64, 9),
+                                   (9, 455, 6)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

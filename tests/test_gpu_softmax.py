@@ -184,7 +184,19 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              (1300, 19, 3), (516, 32, 5), (1028, 2, 3),
              # eight lanes per pixel group (33 to 256 classes with 16-byte accesses), and the streamed kernel beyond
              (20, 48, 3), (20, 64, 2), (24, 65, 2), (24, 128, 2), (24, 129, 2), (16, 200, 2), (8, 256, 3), (520, 40, 2),
-             (8, 300, 2), (5, 257, 3), (64, 1000, 2), (7, 300, 2)]
+             (8, 300, 2), (5, 257, 3), (64, 1000, 2), (7, 300, 2),
+             # planes of 1024 pixels and more never go through the LDS tile: every register and streaming kernel,
+             # 16-byte and 4-byte forms
+             (1028, 8, 2), (1032, 24, 2), (1024, 32, 2), (1028, 33, 2), (1028, 48, 2), (1024, 64, 1), (1032, 65, 2),
+             (1028, 100, 1), (1024, 128, 1), (1028, 129, 1), (1024, 192, 1), (1028, 200, 1), (1024, 256, 2),
+             (1028, 300, 1), (1025, 19, 2), (1025, 40, 2), (1027, 100, 1), (1025, 130, 1), (1025, 257, 1),
+             # the LDS tile (planes that are not whole 64-byte pieces, up to 64 classes, samples up to 32 KB) and
+             # its neighbours: the largest sample and one class more, the longest plane, one sample per tile and
+             # many, sample sizes that are and are not multiples of four floats or of the 32 banks
+             (196, 32, 9), (196, 41, 5), (196, 42, 3), (1023, 8, 3), (1020, 8, 5), (1020, 9, 2), (127, 64, 3),
+             (127, 65, 3), (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 16, 3000), (6, 6, 700), (3, 64, 50),
+             (2, 2, 9000), (2, 1, 5000), (15, 7, 300),
+             (512, 32, 3), (3, 5461, 2), (196, 64, 9), (196, 84, 3), (9, 455, 6), (2, 8192, 3)]
 
 
 @pytest.mark.parametrize("P,C,N", ND_SHAPES)
@@ -222,13 +234,14 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
         assert_bit_exact(host(dxa), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, dx_in=old), "nd bwd acc vs fp32")
 
 
+@pytest.mark.parametrize("P", [8, 1028])
 @pytest.mark.parametrize("C", [3, 19, 40, 100, 200, 300])
-def test_softmax_nd_special_values(oracle, C):
+def test_softmax_nd_special_values(oracle, C, P):
     # register-resident (2 or 8 lanes per pixel group up to 256 classes; one pixel per thread without 16-byte
     # accesses up to 128) and streaming kernels: -inf entries get probability 0, a NaN
     # poisons its pixel only, a pixel of +-1e30 and one of large equal values do not overflow, widely spread logits
-    # keep their small probabilities to the relative bar
-    P, N = 8, 2
+    # keep their small probabilities to the relative bar.  P = 8 goes through the LDS tile up to 64 classes.
+    N = 2
     g = np.random.default_rng(C)
     x = g.standard_normal((N, C, P)).astype(F32)
     x[0, :, 0] = -np.inf
