@@ -243,6 +243,7 @@ struct Tuning {
   Knob reduce_lanes_max_ctiles;  // lane tiles: most channel groups (bounds the grid for very many channels)
   Knob reduce_lanes_min_run;     // lane tiles: fewest contiguous floats a tile reads per sample
   Knob nd_xcd_mask;              // n-d softmax kernels that deal pixel groups per XCD: 1 softmax, 2 NLL backward (default), 4 NLL gather
+  Knob nd_bwd_flat_max_plane;    // n-d NLL backward: planes of up to this many pixels are walked as a flat array
 };
 
 // The streaming mask to use for an array of `bytes` bytes: the load bit of `mask` from nt_min_bytes on, the store

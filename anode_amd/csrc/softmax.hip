@@ -1405,10 +1405,13 @@ void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint3
   note_launch(symbol);
 }
 
-// The same map for planes shorter than 1024 pixels, walked as the flat array it is: a thread takes one 16-byte group
-// of dx (four consecutive pixels of one class), so a wave's accesses are 1 KiB contiguous however short the planes
-// are, and fetches its pixels' dy and labels from the caches (every class of a sample asks for the same ones).
-// [196, 19, 18020]: 3.6 -> 5.5 TB/s.  The arithmetic is that of the kernel above.
+// The same map walked as the flat array it is: a thread takes one 16-byte group of dx (four consecutive pixels of
+// one class), so a wave's accesses are 1 KiB contiguous however short the planes are, and fetches its pixels' dy and
+// labels from the caches (every class of a sample asks for the same ones).  Taken for planes of up to
+// nd_bwd_flat_max_plane pixels (131072: a sample's dy and labels, 8 bytes per pixel, then stay in the L2s while its
+// classes go by): [196, 19, 18020] 3.6 -> 5.6 TB/s, [2048, 64, 512] 4.6 -> 5.8, [65536, 100, 10] 4.9 -> 5.8,
+// accumulating 5.0 -> 6.3; at [524288, 19, 8] inside a softmax -> NLL -> backward sequence it loses to the kernel
+// above, 127 us against 110.  The arithmetic is that of the kernel above.
 template <bool ACC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_kernel(uint32_t P, uint32_t C, uint32_t total_groups,
                                                                              FastDiv div_gpp, FastDiv div_c, uint32_t ignore,
@@ -1467,7 +1470,7 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
   uint32_t chunk = C;
-  if (vec && P < 1024) {
+  if (vec && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
     const uint32_t total_groups = len / 4u;
     const FastDiv div_gpp(P / 4u), div_c(C);
     with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {

@@ -196,7 +196,9 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              (196, 32, 9), (196, 41, 5), (196, 42, 3), (1023, 8, 3), (1020, 8, 5), (1020, 9, 2), (127, 64, 3),
              (127, 65, 3), (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 16, 3000), (6, 6, 700), (3, 64, 50),
              (2, 2, 9000), (2, 1, 5000), (15, 7, 300),
-             (512, 32, 3), (3, 5461, 2), (196, 64, 9), (196, 84, 3), (9, 455, 6), (2, 8192, 3)]
+             (512, 32, 3), (3, 5461, 2), (196, 64, 9), (196, 84, 3), (9, 455, 6), (2, 8192, 3),
+             # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
+             (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
 
 @pytest.mark.parametrize("P,C,N", ND_SHAPES)

@@ -22,6 +22,10 @@ PROFILES = {
     "nontemporal_off": {3: 0, 4: 0},
     "one_workgroup_per_cu": {0: 1},
     "one_workgroup_per_cu_nontemporal": {0: 1, 5: 0},
+    # knob 14: the n-d NLL backward pass walks planes of up to this many pixels as a flat array; 0 sends every shape
+    # to the kernel that gives a thread four pixels and walks their classes (the default only does so from 131073 on)
+    "nd_backward_by_pixel_groups": {14: 0},
+    "nd_backward_by_pixel_groups_nontemporal": {14: 0, 5: 0},
 }
 
 
@@ -56,7 +60,7 @@ def test_softmax_under_tuning(tuned, oracle):
         for name in T_sm.ROW_ENTRY_POINTS:
             T_sm.test_softmax_rows(oracle, name, K, R)
     T_sm.test_softmax_cat_nll_and_bwd_rows(oracle, 1000, 256)
-    for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3)]:
+    for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3), (16, 200, 2), (1024, 256, 2)]:
         T_sm.test_softmax_nd_all_symbols(oracle, P, C, N)
 
 
