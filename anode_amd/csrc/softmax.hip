@@ -1340,6 +1340,200 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
   });
 }
 
+// More classes than the register kernels hold well (from 193 on; from 65 on for planes shorter than 1024 pixels),
+// 16-byte accesses: a workgroup takes a tile of TP consecutive pixels of one sample with all their classes -- C runs
+// of TP floats, one per plane, 32 KB together (up to 59 KB where that is what 32 pixels, or 16 of a short plane,
+// take) -- into LDS, row k of the tile holding plane k's run, 16 bytes per lane both ways.  L = 256 / TP threads
+// share a pixel: thread (j, l) walks classes l, l + L, ... of pixel j (consecutive threads take consecutive pixels:
+// consecutive banks); the L maxima and the L sums of a pixel meet through LDS.  x is read once, where the streaming
+// kernel reads it twice, and a lane holds nothing but its running values, where the register kernel holds 32 values
+// of 16 bytes: [65536, 200] 4.1 -> 4.6 TB/s, [65536, 300] 3.4 -> 3.9, [4096, 300] 3.3 -> 4.4, [1024, 256] 4.3 -> 5.2,
+// [784, 100] 3.2 -> 5.2, [64, 100] 3.3 -> 5.6, [64, 300] 3.2 -> 4.4, [16, 256] 4.6 -> 5.8; [196, 65...300], whose
+// 784-byte planes start anywhere in a line, stay at 2.5-3.5.  (From 65 to 192 classes on long planes the register
+// kernels are faster, 5.0-5.2 against 4.5-5.0.)  Long planes are cut into runs of whole 128-byte lines, short ones
+// into tiles of about the same width.  A pixel's sum is the sum of its L partial sums, each added in class order:
+// the order depends on the shape and on nothing else.  Every entry point (plain, with the label gather, with the
+// backward pass) runs this kernel for these shapes.
+constexpr uint32_t kColTileFloats = 8192;      // the tile a workgroup aims for: four workgroups per CU
+constexpr uint32_t kColTileMaxFloats = 15104;  // the largest tile, 59 KB, beside 5 KB of per-pixel arrays
+
+struct ColTile {
+  uint32_t TP;  // pixels per tile: a multiple of 4, 16 to 256
+  uint32_t L;   // threads per pixel
+  uint32_t tiles_per_sample;
+  bool fits;
+};
+
+ColTile nd_col_tile(uint32_t P, uint32_t C) {
+  ColTile ct = {0, 0, 0, false};
+  if (P % 4u != 0 || P < 16 || C < (P < 1024 ? 65u : 193u)) return ct;
+  uint32_t TP = (kColTileFloats / C) & ~3u;
+  if (TP < 32) TP = (kColTileMaxFloats / C) & ~3u;  // many classes: the largest tile
+  if (TP < 16) return ct;
+  if (TP > 256) TP = 256;
+  if (TP >= P) {
+    TP = P;
+  } else if (P >= 1024) {
+    if (TP < 32) return ct;
+    TP &= ~31u;  // runs of whole 128-byte lines
+  } else {
+    const uint32_t tiles = (P + TP - 1) / TP;  // short planes: tiles of about the same width
+    TP = ((P + tiles - 1) / tiles + 3u) & ~3u;
+  }
+  ct.TP = TP;
+  ct.L = 256u / TP;
+  ct.tiles_per_sample = (P + TP - 1) / TP;
+  ct.fits = true;
+  return ct;
+}
+
+template <bool NLL, bool BWD, int NT>
+__global__ __launch_bounds__(kBlock) void softmax_nd_coltile_kernel(uint32_t P, uint32_t C, uint32_t TP, uint32_t L,
+                                                                    uint32_t total_tiles, FastDiv div_tps,
+                                                                    FastDiv div_tp, uint32_t ignore, uint32_t xcd,
+                                                                    const float *__restrict__ x, float *__restrict__ y,
+                                                                    const uint32_t *__restrict__ cat,
+                                                                    float *__restrict__ nll,
+                                                                    const float *__restrict__ dy,
+                                                                    float *__restrict__ dx) {
+  extern __shared__ __align__(16) float smem[];
+  float *tile = smem;                                          // C rows of TP floats
+  float *part_max = tile + C * TP;                             // [L][TP]
+  float *part_sum = part_max + kBlock;                         // [L][TP]
+  float *inv = part_sum + kBlock;                              // [TP]
+  uint32_t *labs = reinterpret_cast<uint32_t *>(inv + kBlock);  // [TP]
+  float *dys = reinterpret_cast<float *>(labs + kBlock);       // [TP]
+  f32x4 *tile4 = reinterpret_cast<f32x4 *>(tile);
+  const uint32_t row4 = TP / 4u;  // 16-byte groups per tile row
+  uint32_t l, j;                  // this thread's place in the pixel phases
+  div_tp.divmod(threadIdx.x, l, j);
+  // One tile per workgroup (a workgroup that walked several tiles, with the next tile's loads requested before the
+  // current tile's pixel phases, measured slower: [784, 100] 4.1 TB/s against 5.3).  With `xcd` (long planes),
+  // neighbouring tiles run on the same XCD: [1024, 256] 4.7 -> 5.2 TB/s, [4096, 150] 4.7 -> 5.1; on short planes
+  // it loses ([196, 100] 3.5 -> 3.2, [16, 256] 5.8 -> 5.5).
+  for (uint32_t b0 = blockIdx.x; b0 < total_tiles; b0 += gridDim.x) {
+    const uint32_t b = (xcd && gridDim.x == total_tiles) ? xcd_contiguous(b0, total_tiles) : b0;
+    uint32_t n, ti;
+    div_tps.divmod(b, n, ti);
+    const uint32_t p0 = ti * TP;
+    const uint32_t tp = P - p0 < TP ? P - p0 : TP;  // a multiple of 4, as P and TP are
+    const size_t base = size_t(P) * C * n + p0;
+    const size_t pix = size_t(P) * n + p0;
+    if (NLL && threadIdx.x < tp) {
+      const uint32_t label = cat[pix + threadIdx.x];
+      labs[threadIdx.x] = label;
+      if (BWD) dys[threadIdx.x] = (ignore && label >= C) ? 0.0f : dy[pix + threadIdx.x];
+    }
+    // Group q of the tile is group q % ppr of plane q / ppr's run; a thread's groups are 256 apart, so (k, jj) moves
+    // by (256 / ppr, 256 % ppr) with a carry.
+    const uint32_t ppr = tp / 4u, groups = C * ppr;
+    const uint32_t step_k = kBlock / ppr, step_j = kBlock % ppr;
+    const uint32_t k_first = threadIdx.x / ppr, jj_first = threadIdx.x - k_first * ppr;
+    {
+      uint32_t k = k_first, jj = jj_first;
+      // eight groups per thread are requested before the first is written to LDS (a slot past the tile's end reads
+      // the tile's first group again and is dropped)
+      for (uint32_t q0 = 0; q0 < groups; q0 += 8u * kBlock) {
+        f32x4 in[8];
+        uint32_t at[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const bool live = q0 + threadIdx.x + uint32_t(i) * kBlock < groups;
+          at[i] = live ? k * row4 + jj : 0xffffffffu;
+          in[i] = load_stream<NT>(reinterpret_cast<const f32x4 *>(x + base + (live ? size_t(P) * k + 4u * jj : 0)));
+          k += step_k;
+          jj += step_j;
+          if (jj >= ppr) {
+            jj -= ppr;
+            ++k;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (at[i] != 0xffffffffu) tile4[at[i]] = in[i];
+        }
+      }
+    }
+    __syncthreads();
+    const bool active = l < L && j < tp;
+    float m = kNegInf;
+    if (active) {
+#pragma unroll 4
+      for (uint32_t k = l; k < C; k += L) m = fmaxf(m, tile[k * TP + j]);
+      part_max[l * TP + j] = m;
+    }
+    __syncthreads();
+    if (active) {
+      for (uint32_t ll = 0; ll < L; ++ll) m = fmaxf(m, part_max[ll * TP + j]);
+      float sum = 0.0f;
+#pragma unroll 4
+      for (uint32_t k = l; k < C; k += L) {
+        const float e = exp_nonpos(tile[k * TP + j] - m);
+        tile[k * TP + j] = e;
+        sum += e;
+      }
+      part_sum[l * TP + j] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x < tp) {
+      float sum = part_sum[threadIdx.x];
+      for (uint32_t ll = 1; ll < L; ++ll) sum += part_sum[ll * TP + threadIdx.x];
+      const float r = 1.0f / sum;  // one correctly rounded reciprocal per pixel
+      inv[threadIdx.x] = r;
+      if (NLL) {
+        // -log of the stored probability of the label; NaN (0 with `ignore`) when the label is out of range
+        const uint32_t label = labs[threadIdx.x];
+        nll[pix + threadIdx.x] =
+            label < C ? -logf(tile[label * TP + threadIdx.x] * r) : (ignore ? 0.0f : __builtin_nanf(""));
+      }
+    }
+    __syncthreads();
+    {
+      uint32_t k = k_first, jj = jj_first;
+      for (uint32_t q = threadIdx.x; q < groups; q += kBlock) {
+        const f32x4 e = tile4[k * row4 + jj];
+        const f32x4 r = reinterpret_cast<const f32x4 *>(inv)[jj];
+        const f32x4 pr = {e.x * r.x, e.y * r.y, e.z * r.z, e.w * r.w};
+        const size_t off = base + size_t(P) * k + 4u * jj;
+        store_stream<NT>(reinterpret_cast<f32x4 *>(y + off), pr);
+        if (BWD) {
+          const u32x4 lab = reinterpret_cast<const u32x4 *>(labs)[jj];
+          const f32x4 d = reinterpret_cast<const f32x4 *>(dys)[jj];
+          f32x4 gr;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) gr[w] = d[w] * (pr[w] - float(lab[w] == k));
+          store_stream<NT>(reinterpret_cast<f32x4 *>(dx + off), gr);
+        }
+        k += step_k;
+        jj += step_j;
+        if (jj >= ppr) {
+          jj -= ppr;
+          ++k;
+        }
+      }
+    }
+    __syncthreads();  // the next tile overwrites all of it
+  }
+}
+
+template <bool NLL, bool BWD>
+void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
+                               const uint32_t *cat, float *nll, const float *dy, float *dx, bool ignore,
+                               hipStream_t s) {
+  const uint32_t total_tiles = ct.tiles_per_sample * N;  // at most len / 16
+  const uint32_t max_blocks = 1u << 24;
+  const uint32_t blocks = total_tiles < max_blocks ? total_tiles : max_blocks;
+  const size_t lds_bytes = (size_t(C) * ct.TP + 5u * kBlock) * sizeof(float);
+  const FastDiv div_tps(ct.tiles_per_sample), div_tp(ct.TP);
+  const uint32_t xcd = P >= 1024 ? 1u : 0u;
+  // logits in, probabilities (and the gradient) out: all streamed
+  const int nt = stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal);
+  with_stream_policy(nt, [&](auto policy) {
+    softmax_nd_coltile_kernel<NLL, BWD, decltype(policy)::value><<<blocks, kBlock, lds_bytes, s>>>(
+        P, C, ct.TP, ct.L, total_tiles, div_tps, div_tp, ignore ? 1u : 0u, xcd, x, y, cat, nll, dy, dx);
+  });
+}
+
 // Which kernel takes 33 to 128 classes: one pixel per thread where 16-byte accesses are not legal, or where the
 // planes are so short that eight lanes per pixel group would read 128-byte pieces of them (P = 196, C = 64:
 // 3.7 TB/s against 2.3).  The plain and the fused entry points must agree on this: the order in which a pixel's
@@ -1356,8 +1550,11 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
   }
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
+  const ColTile ct = nd_col_tile(P, C);
   if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+  } else if (vec && ct.fits) {
+    launch_softmax_nd_coltile<false, false>(ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (nd_one_pixel_per_thread(P, C, vec)) {
     // one pixel per thread keeps
     // the row in registers and is still coalesced across the wave
@@ -1591,6 +1788,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                         as_stream(stream));
     note_launch(__func__);
+  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0); ct.fits && aligned16(x) && aligned16(softmax)) {
+    launch_softmax_nd_coltile<true, false>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
+                                           false, as_stream(stream));
+    note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll);
              dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
@@ -1623,6 +1824,11 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   } else if (nd_tile_fits(prefix_dim, dim0)) {
     launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                        as_stream(stream));
+    note_launch(__func__);
+  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0);
+             ct.fits && aligned16(x) && aligned16(softmax) && aligned16(dx)) {
+    launch_softmax_nd_coltile<true, true>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
+                                          as_stream(stream));
     note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll) && aligned16(dy) && aligned16(dx);

@@ -194,7 +194,9 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
                                    # short planes through the LDS tile, and its neighbours
                                    (196, 32, 9), (196, 41, 5), (196, 42, 3), (1023, 8, 3), (127, 64, 3), (127, 65, 3),
                                    (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 2, 9000), (512, 32, 3), (196, 64, 9),
-                                   (9, 455, 6)])
+                                   (9, 455, 6),
+                                   # tiles of all classes of a run of pixels in LDS
+                                   (64, 300, 3), (196, 150, 2), (1028, 200, 1), (20, 70, 5), (16, 944, 1), (1056, 256, 2)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

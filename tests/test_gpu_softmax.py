@@ -197,6 +197,11 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              (127, 65, 3), (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 16, 3000), (6, 6, 700), (3, 64, 50),
              (2, 2, 9000), (2, 1, 5000), (15, 7, 300),
              (512, 32, 3), (3, 5461, 2), (196, 64, 9), (196, 84, 3), (9, 455, 6), (2, 8192, 3),
+             # tiles of all classes of a run of pixels in LDS (from 193 classes on, from 65 on planes under 1024 pixels):
+             # ragged last tiles, one tile per plane, 16 to 256 pixels per tile, the largest class counts that fit
+             # (472, 944) and one more
+             (64, 300, 3), (16, 900, 2), (16, 944, 1), (16, 945, 1), (784, 100, 2), (196, 150, 2), (2048, 472, 1),
+             (2048, 473, 1), (20, 70, 5), (256, 65, 2), (1024, 193, 1), (1056, 200, 2), (1000, 65, 2),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
