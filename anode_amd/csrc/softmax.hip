@@ -1348,8 +1348,7 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
 // consecutive banks); the L maxima and the L sums of a pixel meet through LDS.  x is read once, where the streaming
 // kernel reads it twice, and a lane holds nothing but its running values, where the register kernel holds 32 values
 // of 16 bytes: [65536, 200] 4.1 -> 4.6 TB/s, [65536, 300] 3.4 -> 3.9, [4096, 300] 3.3 -> 4.4, [1024, 256] 4.3 -> 5.2,
-// [784, 100] 3.2 -> 5.2, [64, 100] 3.3 -> 5.6, [64, 300] 3.2 -> 4.4, [16, 256] 4.6 -> 5.8; [196, 65...300], whose
-// 784-byte planes start anywhere in a line, stay at 2.5-3.5.  (From 65 to 192 classes on long planes the register
+// [784, 100] 3.2 -> 5.2, [64, 100] 3.3 -> 5.6, [64, 300] 3.2 -> 4.4, [16, 256] 4.6 -> 5.8.  (From 65 to 192 classes on long planes the register
 // kernels are faster, 5.0-5.2 against 4.5-5.0.)  Long planes are cut into runs of whole 128-byte lines, short ones
 // into tiles of about the same width.  A pixel's sum is the sum of its L partial sums, each added in class order:
 // the order depends on the shape and on nothing else.  Every entry point (plain, with the label gather, with the
@@ -1377,7 +1376,11 @@ ColTile nd_col_tile(uint32_t P, uint32_t C) {
     if (TP < 32) return ct;
     TP &= ~31u;  // runs of whole 128-byte lines
   } else {
-    const uint32_t tiles = (P + TP - 1) / TP;  // short planes: tiles of about the same width
+    // Short planes: tiles of about the same width.  Planes that are not whole 32-byte pieces are left to the other
+    // kernels unless a tile holds a whole plane: their runs start anywhere in a piece, and cut runs then share
+    // pieces with their neighbours ([196, 128] 2.5 TB/s against 3.5).
+    if (P % 8u != 0) return ct;
+    const uint32_t tiles = (P + TP - 1) / TP;
     TP = ((P + tiles - 1) / tiles + 3u) & ~3u;
   }
   ct.TP = TP;
