@@ -416,10 +416,22 @@ __global__ __launch_bounds__(THREADS) void softmax_row_blockreg_kernel(uint32_t 
 // one row at a time leaves the memory system idle between the phases; two workgroups overlap them.)
 constexpr int kRowStreamThreads = 512;
 constexpr int kRowStreamHeld = 32 * kRowStreamThreads;  // values of a row that stay in LDS
-template <bool VEC, int NT>
-__global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(uint32_t K, uint32_t R,
+// MODE 0: 4-byte accesses.  MODE 1: 16-byte accesses, every row starts on a 16-byte boundary.  MODE 2: 16-byte
+// accesses to the aligned groups of the array from the start of the 128-byte line of y in which a row begins (x and
+// y, and dx, start equally far from a 16-byte boundary; `mis` is y's distance in floats from a line): every step of
+// a wave then covers whole lines of y, whatever the row length, and the values of a row's first and last groups
+// that belong to its neighbours are read, count as -inf and are not written (such a group is stored value by
+// value).  `unit` is 32 floats, a line, where x lies in its line as y does in its own, and otherwise 4, one group:
+// no load then reaches further back than the 16-byte group in which x begins.  Rows whose ends cut 64-byte pieces in two otherwise cost a fifth of the bandwidth: the two halves of a
+// piece are written by different store instructions.  The order of a row's sum depends on where in a line the row
+// starts.
+// (four waves per SIMD, i.e. at most 128 registers: two workgroups must fit a CU)
+template <int MODE, int NT>
+__global__ __launch_bounds__(kRowStreamThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void softmax_row_stream_kernel(uint32_t K, uint32_t R, uint32_t mis,
+                                                                               uint32_t unit,
                                                                                const float *__restrict__ x,
                                                                                float *__restrict__ y, RowNll nl) {
+  constexpr bool VEC = MODE != 0;
   constexpr int THREADS = kRowStreamThreads;
   constexpr int W = VEC ? 4 : 1;
   constexpr int U = VEC ? 4 : 8;
@@ -429,33 +441,70 @@ __global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(u
   static_assert(kHeldBatches * kBatch * W == uint32_t(kRowStreamHeld), "whole batches are held");
   __shared__ __align__(16) float held[kRowStreamHeld];
   __shared__ float lds_m[WAVES], lds_s[WAVES];
-  const uint32_t groups = K / uint32_t(W);  // VEC: the host checked K % 4 == 0
-  const uint32_t batches = uint32_t((uint64_t(groups) + kBatch - 1u) / kBatch);
-  const uint32_t held_batches = batches < kHeldBatches ? batches : kHeldBatches;
+  // A row's geometry: the `shift` values before it in its line come first (MODE 2 only), `groups` groups reach to
+  // the row's end; group g holds the row's values 4 g - shift ... 4 g - shift + 3.
+  struct RowGeom {
+    const float *xa;  // the row's first group
+    uint32_t shift, groups, batches, held_batches;
+  };
+  auto geom = [&](uint64_t r) {
+    RowGeom g;
+    g.shift = MODE == 2 ? uint32_t((uint64_t(mis) + r * K) & (unit - 1u)) : 0u;
+    g.xa = x + size_t(r) * K - g.shift;
+    g.groups = MODE == 2 ? uint32_t((uint64_t(K) + g.shift + 3u) / 4u) : K / uint32_t(W);  // MODE 1: K % 4 == 0
+    g.batches = uint32_t((uint64_t(g.groups) + kBatch - 1u) / kBatch);
+    g.held_batches = g.batches < kHeldBatches ? g.batches : kHeldBatches;
+    return g;
+  };
+  // The values of group g that are the row's: j_lo <= j < j_hi.  (None for a group past the row's end; in MODE 2
+  // the first groups hold the `shift` values before the row, and the last group may end with values of the row
+  // after.)
+  struct InRow {
+    uint32_t j_lo, j_hi;
+    __device__ bool operator()(int j) const { return uint32_t(j) >= j_lo && uint32_t(j) < j_hi; }
+    __device__ bool none() const { return j_lo >= j_hi; }
+    __device__ bool all() const { return j_lo == 0u && j_hi == uint32_t(W); }
+  };
+  auto in_row = [&](const RowGeom &rg, uint64_t g) {
+    InRow v;
+    if (MODE != 2) {
+      v.j_lo = 0u;
+      v.j_hi = g < rg.groups ? uint32_t(W) : 0u;
+    } else {
+      const uint64_t first = g * 4u, end = uint64_t(K) + rg.shift;  // in values counted from the line's start
+      v.j_lo = first >= rg.shift ? 0u : (rg.shift - first < 4u ? uint32_t(rg.shift - first) : 4u);
+      v.j_hi = first >= end ? 0u : (end - first < 4u ? uint32_t(end - first) : 4u);
+    }
+    return v;
+  };
+  // every value of group g is the row's (MODE 2)
+  auto inside = [&](const RowGeom &rg, uint64_t g) { return g * 4u >= rg.shift && g * 4u + 4u <= uint64_t(K) + rg.shift; };
   // 64-bit group numbers: a batch's first group plus the batch can pass 2^32.  A batch past the row's end is
   // requested like any other (it reads the row's last group) and counts for nothing.
-  auto request = [&](const float *xr, uint32_t b, float (&t)[U][W], auto last_use) {
+  auto request = [&](const RowGeom &rg, uint32_t b, float (&t)[U][W], auto last_use) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint64_t g = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x;
-      const uint32_t gc = g < groups ? uint32_t(g) : groups - 1u;
+      const uint32_t gc = g < rg.groups ? uint32_t(g) : rg.groups - 1u;
       if (VEC) {
-        const f32x4 q = decltype(last_use)::value ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + size_t(gc) * 4u))
-                                                  : *reinterpret_cast<const f32x4 *>(xr + size_t(gc) * 4u);
+        const f32x4 q = decltype(last_use)::value ? load_stream<NT>(reinterpret_cast<const f32x4 *>(rg.xa + size_t(gc) * 4u))
+                                                  : *reinterpret_cast<const f32x4 *>(rg.xa + size_t(gc) * 4u);
 #pragma unroll
         for (int j = 0; j < W; ++j) t[u][j] = q[j];
       } else {
-        t[u][0] = xr[gc];
+        t[u][0] = rg.xa[gc];
       }
     }
   };
   float ta[U][W], tb[U][W];
-  if (blockIdx.x < R) request(x + size_t(blockIdx.x) * K, 0, ta, std::false_type{});
+  RowGeom rg = geom(blockIdx.x < R ? blockIdx.x : 0u);
+  if (blockIdx.x < R) request(rg, 0, ta, std::false_type{});
   for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
-    const float *xr = x + size_t(r) * K;
-    float *yr = y + size_t(r) * K;
+    float *ya = y + size_t(r) * K - rg.shift;
+    float *dxa = (nl.on() && nl.dx != nullptr) ? nl.dx + size_t(r) * K - rg.shift : nullptr;
     const uint32_t label = nl.on() ? nl.label(r) : 0u;
     const float dyr = (nl.on() && nl.dx != nullptr) ? nl.dy[r] : 0.0f;
+    const uint32_t batches = rg.batches, held_batches = rg.held_batches;
     // the held batches: slot (b * U + u) * THREADS + threadIdx.x, written and read by the same thread
     auto keep = [&](uint32_t b, const float (&t)[U][W]) {
       if (b >= held_batches) return;
@@ -487,11 +536,18 @@ __global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(u
       float bm = kNegInf;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const bool in = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x < groups;
+        const uint64_t g = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x;
+        // MODE 2: a wave whose groups all lie inside the row (all but the waves at a row's two ends) masks nothing
+        if (MODE == 2 && __all(inside(rg, g))) {
 #pragma unroll
-        for (int j = 0; j < W; ++j) {
-          if (!in) t[u][j] = kNegInf;
-          bm = fmaxf(bm, t[u][j]);
+          for (int j = 0; j < W; ++j) bm = fmaxf(bm, t[u][j]);
+        } else {
+          const InRow mine = in_row(rg, g);
+#pragma unroll
+          for (int j = 0; j < W; ++j) {
+            if (!mine(j)) t[u][j] = kNegInf;
+            bm = fmaxf(bm, t[u][j]);
+          }
         }
       }
       float bs = 0.0f;
@@ -523,24 +579,43 @@ __global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(u
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint64_t g = uint64_t(b) * kBatch + uint32_t(u) * uint32_t(THREADS) + threadIdx.x;
-        if (g < groups) {
-          const uint32_t k = uint32_t(g) * uint32_t(W);
+        InRow mine;
+        if (MODE == 2 && __all(inside(rg, g))) {
+          mine.j_lo = 0u;
+          mine.j_hi = uint32_t(W);
+        } else {
+          mine = in_row(rg, g);
+        }
+        if (!mine.none()) {
+          // the row's value number of the group's first value; "negative" (wrapped) for the values of a first group
+          // that belong to the row before, which `mine` leaves out
+          const uint32_t k = uint32_t(g) * uint32_t(W) - rg.shift;
 #pragma unroll
           for (int j = 0; j < W; ++j) {
             t[u][j] = exp_nonpos(t[u][j] - m) * rs;
-            if (nl.on()) nl.emit_nll(r, K, label, k + uint32_t(j), t[u][j]);
+            if (nl.on() && mine(j)) nl.emit_nll(r, K, label, k + uint32_t(j), t[u][j]);
           }
           if (VEC) {
-            store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{t[u][0], t[u][1], t[u][2], t[u][3]});
-            if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
-              store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
-                               f32x4{RowNll::grad(dyr, label, k, t[u][0]), RowNll::grad(dyr, label, k + 1u, t[u][1]),
-                                     RowNll::grad(dyr, label, k + 2u, t[u][2]),
-                                     RowNll::grad(dyr, label, k + 3u, t[u][3])});
+            if (mine.all()) {
+              store_stream<NT>(reinterpret_cast<f32x4 *>(ya + size_t(g) * 4u), f32x4{t[u][0], t[u][1], t[u][2], t[u][3]});
+              if (dxa != nullptr) {  // the host checked that dx lies like y
+                store_stream<NT>(reinterpret_cast<f32x4 *>(dxa + size_t(g) * 4u),
+                                 f32x4{RowNll::grad(dyr, label, k, t[u][0]), RowNll::grad(dyr, label, k + 1u, t[u][1]),
+                                       RowNll::grad(dyr, label, k + 2u, t[u][2]),
+                                       RowNll::grad(dyr, label, k + 3u, t[u][3])});
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < W; ++j) {
+                if (mine(j)) {
+                  ya[size_t(g) * 4u + uint32_t(j)] = t[u][j];
+                  if (dxa != nullptr) dxa[size_t(g) * 4u + uint32_t(j)] = RowNll::grad(dyr, label, k + uint32_t(j), t[u][j]);
+                }
+              }
             }
           } else {
-            yr[k] = t[u][0];
-            if (nl.on() && nl.dx != nullptr) nl.dx[size_t(r) * K + k] = RowNll::grad(dyr, label, k, t[u][0]);
+            ya[g] = t[u][0];
+            if (dxa != nullptr) dxa[g] = RowNll::grad(dyr, label, k, t[u][0]);
           }
         }
       }
@@ -549,10 +624,10 @@ __global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(u
     // previous row before it began to store
 #pragma unroll 1
     for (uint32_t b = 0; b < batches; b += 2) {
-      request(xr, b + 1u, tb, std::false_type{});
+      request(rg, b + 1u, tb, std::false_type{});
       fold(b, ta);
       keep(b, ta);
-      request(xr, b + 2u, ta, std::false_type{});
+      request(rg, b + 2u, ta, std::false_type{});
       fold(b + 1u, tb);
       keep(b + 1u, tb);
     }
@@ -574,22 +649,24 @@ __global__ __launch_bounds__(kRowStreamThreads) void softmax_row_stream_kernel(u
     __syncthreads();
     rs = 1.0f / s;
     if (held_batches < batches) {
-      request(xr, held_batches, ta, std::true_type{});
+      request(rg, held_batches, ta, std::true_type{});
 #pragma unroll 1
       for (uint32_t b = held_batches; b < batches; b += 2) {
-        request(xr, b + 1u, tb, std::true_type{});
+        request(rg, b + 1u, tb, std::true_type{});
         write(b, ta);
-        request(xr, b + 2u, ta, std::true_type{});
+        request(rg, b + 2u, ta, std::true_type{});
         write(b + 1u, tb);
       }
     }
     // the next row starts to arrive while this one's held part is written
-    if (r + gridDim.x < R) request(x + size_t(r + gridDim.x) * K, 0, ta, std::false_type{});
+    const RowGeom next = geom(r + gridDim.x < R ? r + gridDim.x : r);
+    if (r + gridDim.x < R) request(next, 0, ta, std::false_type{});
 #pragma unroll 1
     for (uint32_t b = 0; b < held_batches; ++b) {
       recall(b, tb);
       write(b, tb);
     }
+    rg = next;
   }
 }
 
@@ -713,12 +790,24 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       // two workgroups per CU, which walk their rows
       const uint32_t cus = 2u * uint32_t(device_cu_count());
       const uint32_t walkers = R < cus ? R : cus;
+      // Rows that do not start on 128-byte lines are read and written in the array's 16-byte groups, from the
+      // start of y's line, where x and y (and dx) start equally far from a 16-byte boundary.
+      const auto floats_past = [](const float *p, uint32_t unit) { return uint32_t((reinterpret_cast<uintptr_t>(p) >> 2) & (unit - 1u)); };
+      const auto lies_like_y = [&](const float *p) { return floats_past(p, 4) == floats_past(y, 4); };
+      const bool floats = (reinterpret_cast<uintptr_t>(x) & 3u) == 0 && (reinterpret_cast<uintptr_t>(y) & 3u) == 0;
       if (vec) {
         with_stream_policy(nt, [&](auto policy) {
-          softmax_row_stream_kernel<true, decltype(policy)::value><<<walkers, kRowStreamThreads, 0, s>>>(K, R, x, y, nl);
+          softmax_row_stream_kernel<1, decltype(policy)::value>
+              <<<walkers, kRowStreamThreads, 0, s>>>(K, R, 0u, 1u, x, y, nl);
+        });
+      } else if (floats && lies_like_y(x) && (nl.dx == nullptr || lies_like_y(nl.dx))) {
+        const uint32_t unit = floats_past(x, 32) == floats_past(y, 32) ? 32u : 4u;
+        with_stream_policy(nt, [&](auto policy) {
+          softmax_row_stream_kernel<2, decltype(policy)::value>
+              <<<walkers, kRowStreamThreads, 0, s>>>(K, R, floats_past(y, unit), unit, x, y, nl);
         });
       } else {
-        softmax_row_stream_kernel<false, 0><<<walkers, kRowStreamThreads, 0, s>>>(K, R, x, y, nl);
+        softmax_row_stream_kernel<0, 0><<<walkers, kRowStreamThreads, 0, s>>>(K, R, 0u, 1u, x, y, nl);
       }
     }
 #undef ANODE_ROW_BLOCKREG

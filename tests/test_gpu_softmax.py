@@ -143,6 +143,46 @@ def test_softmax_long_rows_special_values(oracle, K):
         assert not np.any(np.isnan(p[[0, 1, 2, 3, 5, 6, 7]]))
 
 
+@pytest.mark.parametrize("K,R", [(32773, 5), (50257, 3), (40002, 4), (65536, 3)])
+def test_softmax_long_rows_touch_nothing_but_their_rows(oracle, K, R):
+    # Long rows that do not start on 16-byte boundaries are read and written in the array's 16-byte groups where x
+    # and y start equally far from such a boundary: the groups at a row's ends are shared with its neighbours, and
+    # with whatever lies before and after the array.  Guard bands around y must come back untouched, for every
+    # distance from a boundary, and also where x and y lie differently (4-byte accesses).
+    import torch
+    g = np.random.default_rng(K + R)
+    x = (2 * g.standard_normal(K * R)).astype(F32)
+    want = oracle.softmax(K, R, x, f64=True)
+    lab = g.integers(0, K, R).astype(np.uint32)
+    dy = g.standard_normal(R).astype(F32)
+    # (x and y alike within a 16-byte group but not within a 128-byte line: (1, 5), (3, 31))
+    for off_x, off_y in [(0, 0), (1, 1), (2, 2), (3, 3), (1, 2), (0, 3), (1, 5), (3, 31)]:
+        print(f"case long rows K={K} R={R} x+{off_x} y+{off_y}", flush=True)
+        buf = torch.full((K * R + 64,), 12345.0, dtype=torch.float32, device="cuda")
+        y = buf[16 + off_y:16 + off_y + K * R]
+        # what lies before and after x must not count: NaN there would reach every probability of the row
+        xbuf = torch.full((K * R + 64,), float("nan"), dtype=torch.float32, device="cuda")
+        xd = xbuf[16 + off_x:16 + off_x + K * R]
+        xd.copy_(torch.from_numpy(x))
+        call("anode_gpu_softmax_packed_deterministic_f32", K, R, xd, y)
+        whole = host(buf)
+        assert np.all(whole[:16 + off_y] == 12345.0) and np.all(whole[16 + off_y + K * R:] == 12345.0)
+        assert_close(whole[16 + off_y:16 + off_y + K * R], want, f"softmax K={K} x+{off_x} y+{off_y}", abs_floor=1e-30)
+        # softmax + NLL + backward in one launch: dx lies like y
+        buf2 = torch.full((K * R + 64,), 12345.0, dtype=torch.float32, device="cuda")
+        dbuf = torch.full((K * R + 64,), 54321.0, dtype=torch.float32, device="cuda")
+        y2, dx = buf2[16 + off_y:16 + off_y + K * R], dbuf[16 + off_y:16 + off_y + K * R]
+        nll = empty(R)
+        call("anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32", K, R, xd, dev(lab), dev(dy), y2, nll, dx)
+        whole2, wholed = host(buf2), host(dbuf)
+        assert np.all(whole2[:16 + off_y] == 12345.0) and np.all(whole2[16 + off_y + K * R:] == 12345.0)
+        assert np.all(wholed[:16 + off_y] == 54321.0) and np.all(wholed[16 + off_y + K * R:] == 54321.0)
+        assert_bit_exact(whole2[16 + off_y:16 + off_y + K * R], whole[16 + off_y:16 + off_y + K * R], "fused p")
+        p = whole2[16 + off_y:16 + off_y + K * R]
+        assert_bit_exact(wholed[16 + off_y:16 + off_y + K * R], oracle.softmax_cat_nll_bwd(K, R, dy, p, lab), "fused dx")
+        assert_close(host(nll), oracle.softmax_cat_nll(K, R, p, lab, f64=True), "fused nll", abs_floor=1e-6)
+
+
 @pytest.mark.parametrize("K,R", [(10, 32), (1000, 256), (7, 5), (1, 9), (300, 11)])
 def test_softmax_cat_nll_and_bwd_rows(oracle, K, R):
     g = np.random.default_rng(K + R)
