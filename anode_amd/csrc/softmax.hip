@@ -775,8 +775,18 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       ANODE_ROW_BLOCKREG(16);
     } else if (K <= 8192) {
       ANODE_ROW_BLOCKREG(32);
-    } else if (K <= 16384) {
+    } else if (K <= 9216) {
       ANODE_ROW_BLOCKREG(64);
+    } else if (K <= 16384) {
+      // workgroups of 512 threads, 32 values each: two to a CU with four waves per SIMD, where 256 threads of 64
+      // values leave two ([4096, 16384] 5.2 -> 5.6 TB/s, [5460, 12289] 4.3 -> 5.0; [8188, 8196] 5.8 against 5.6)
+      if (vec) {
+        with_stream_policy(nt, [&](auto policy) {
+          softmax_row_blockreg_kernel<32, true, decltype(policy)::value, 512><<<blocks, 512, 0, s>>>(K, R, x, y, nl);
+        });
+      } else {
+        softmax_row_blockreg_kernel<32, false, 0, 512><<<blocks, 512, 0, s>>>(K, R, x, y, nl);
+      }
     } else if (K <= 32768) {
       // workgroups of 1024 threads, 32 values each
       if (vec) {

@@ -229,7 +229,7 @@ ROW_FUSED_SHAPES = [(1, 5), (2, 7), (10, 32), (19, 513), (32, 600), (33, 9), (64
                     (40, 700), (130, 77), (208, 70), (209, 70), (212, 40), (36, 300), (92, 64), (180, 41), (225, 33), (240, 9),
                     (250, 21), (256, 33), (1012, 19), (2052, 11), (4100, 9),
                     (1000, 256), (1024, 3), (1025, 2), (2048, 2), (2049, 3), (4097, 2), (16385, 1), (40000, 1),
-                    (20000, 3), (32768, 2), (32772, 2), (50257, 2), (65540, 3),
+                    (9216, 2), (9220, 2), (12289, 2), (20000, 3), (32768, 2), (32772, 2), (50257, 2), (65540, 3),
                     (32772, 1100)]   # several rows per workgroup of the streaming kernel
 
 

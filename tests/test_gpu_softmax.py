@@ -58,6 +58,8 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (212, 40), (1012, 19), (2044, 9), (2052, 11), (4100, 9), (8196, 3),
               # the limits of the workgroup-per-row register kernel
               (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1),
+              # ... and of its 512-thread form (rows of 9217 to 16384 classes)
+              (9216, 2), (9217, 2), (9220, 3), (12289, 3), (16380, 2),
               # workgroups of 1024 threads: rows in registers up to 32768 classes, streamed twice beyond
               (16388, 3), (20000, 3), (32764, 2), (32768, 2), (32769, 1), (32772, 3), (50257, 2), (65536, 2),
               (65540, 1), (100003, 1), (262148, 2),
