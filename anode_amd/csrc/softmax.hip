@@ -775,7 +775,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       ANODE_ROW_BLOCKREG(16);
     } else if (K <= 8192) {
       ANODE_ROW_BLOCKREG(32);
-    } else if (K <= 9216) {
+    } else if (K <= (vec ? 9216u : 8192u)) {  // (with 4-byte accesses 64 values per thread take 210 registers: [8191, 8193] 3.7 TB/s)
       ANODE_ROW_BLOCKREG(64);
     } else if (K <= 16384) {
       // workgroups of 512 threads, 32 values each: two to a CU with four waves per SIMD, where 256 threads of 64

@@ -145,9 +145,12 @@ def test_softmax_long_rows_special_values(oracle, K):
         assert not np.any(np.isnan(p[[0, 1, 2, 3, 5, 6, 7]]))
 
 
-@pytest.mark.parametrize("K,R", [(32773, 5), (50257, 3), (40002, 4), (65536, 3)])
+@pytest.mark.parametrize("K,R", [(32773, 5), (50257, 3), (40002, 4), (65536, 3),
+                                 # rows in registers: every workgroup size, and the longest row that fits each
+                                 (2050, 5), (4062, 3), (4063, 3), (8158, 2), (8159, 2), (12289, 3), (16350, 2), (16351, 2),
+                                 (30522, 2), (32734, 2), (32735, 2)])
 def test_softmax_long_rows_touch_nothing_but_their_rows(oracle, K, R):
-    # Long rows that do not start on 16-byte boundaries are read and written in the array's 16-byte groups where x
+    # Rows of more than 2048 classes that do not start on 16-byte boundaries are read and written in the array's 16-byte groups where x
     # and y start equally far from such a boundary: the groups at a row's ends are shared with its neighbours, and
     # with whatever lies before and after the array.  Guard bands around y must come back untouched, for every
     # distance from a boundary, and also where x and y lie differently (4-byte accesses).
