@@ -918,14 +918,11 @@ __device__ inline f32x4 lane_swap(f32x4 v, int off) {
 // what the separate gather returns.
 // With BWD the gradient of the summed loss for a dy known up front is written in the same pass:
 // dx = dy * (p - onehot), the arithmetic (and, with pg.ignore, the masking) of softmax_nd_cat_nll_bwd_kernel.
-// (With the backward pass the 20-class form takes 129 registers, one more than four waves per SIMD leave, and the
-// 24-class form with the label gather 130: they are held to 128, [512K, 19, 8] forward + backward 202 -> 178 us.
-// Five waves for the plain 20-class form, 96 registers with 14 values spilled, lose: 137 us against 117.)
-constexpr int nd_reg_min_waves(int cmax, int w, bool nll, bool bwd) {
-  return (w == 4 && ((cmax == 20 && bwd) || (cmax == 24 && nll && !bwd))) ? 4 : 1;
-}
+// (With the backward pass the 20-class form takes 129 registers, one more than four waves per SIMD leave.  Held to
+// 128 it measures the same, 182 us at [512K, 19, 8] in a process that holds nothing else, 204 against 201 among
+// the other arrays of the benchmark: the kernel waits for memory, not for a free wave slot.)
 template <int CMAX, typename V, bool NLL, int NT, int SPLIT, bool BWD = false>
-__global__ __launch_bounds__(kBlock, nd_reg_min_waves(CMAX, PixVec<V>::W, NLL, BWD)) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
+__global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, const float *__restrict__ x,
                                                                 float *__restrict__ y,
                                                                 const uint32_t *__restrict__ cat,
                                                                 float *__restrict__ nll,
