@@ -201,7 +201,10 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
       }
       __syncthreads();
       float *dt = nl.dx + r0 * K;
-      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, tile4[g]);
+      const uint32_t ad = vec ? uint32_t((reinterpret_cast<uintptr_t>(dt) >> 4) & 7u) : 0u;
+      for (uint32_t slot = threadIdx.x; slot < n4 + ad; slot += kBlock) {
+        if (slot >= ad) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + (slot - ad), tile4[slot - ad]);
+      }
       for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) dt[e] = tile[e];
       __syncthreads();
     }
@@ -1343,17 +1346,22 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
     float *yt = y + n0 * slab;
     // eight groups per thread are requested before the first is written to LDS (a slot past the tile's end reads
     // its last group again and is dropped)
-    for (uint32_t g0 = 0; g0 < n4; g0 += 8u * kBlock) {
+    // A wave's step covers whole 128-byte lines of the array: the groups are taken `ax` places later, ax = the
+    // tile's distance in groups from the line before it, so that the first wave's first step is the short one
+    // (a sample of 19 planes of 196 pixels starts anywhere in a line; [196, 19] 4.9 -> 5.2 TB/s, [49, 19] 4.8 -> 5.3).
+    const uint32_t ax = vec ? uint32_t((reinterpret_cast<uintptr_t>(xt) >> 4) & 7u) : 0u;
+    for (uint32_t g0 = 0; g0 < n4 + ax; g0 += 8u * kBlock) {
       f32x4 in[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const uint32_t g = g0 + threadIdx.x + uint32_t(i) * kBlock;
+        const uint32_t slot = g0 + threadIdx.x + uint32_t(i) * kBlock;
+        const uint32_t g = slot >= ax ? slot - ax : 0u;
         in[i] = load_stream<NT>(reinterpret_cast<const f32x4 *>(xt) + (g < n4 ? g : n4 - 1u));
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const uint32_t g = g0 + threadIdx.x + uint32_t(i) * kBlock;
-        if (g < n4) tile4[g] = in[i];
+        const uint32_t slot = g0 + threadIdx.x + uint32_t(i) * kBlock;
+        if (slot >= ax && slot - ax < n4) tile4[slot - ax] = in[i];
       }
     }
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) tile[e] = xt[e];
@@ -1393,7 +1401,10 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
       }
     }
     __syncthreads();
-    for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + g, tile4[g]);
+    const uint32_t ay = vec ? uint32_t((reinterpret_cast<uintptr_t>(yt) >> 4) & 7u) : 0u;
+    for (uint32_t slot = threadIdx.x; slot < n4 + ay; slot += kBlock) {
+      if (slot >= ay) store_stream<NT>(reinterpret_cast<f32x4 *>(yt) + (slot - ay), tile4[slot - ay]);
+    }
     for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) yt[e] = tile[e];
     __syncthreads();  // the tile is overwritten below, or by the next pass
     if (BWD) {
@@ -1409,7 +1420,10 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
       }
       __syncthreads();
       float *dt = dx + n0 * slab;
-      for (uint32_t g = threadIdx.x; g < n4; g += kBlock) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + g, tile4[g]);
+      const uint32_t ad = vec ? uint32_t((reinterpret_cast<uintptr_t>(dt) >> 4) & 7u) : 0u;
+      for (uint32_t slot = threadIdx.x; slot < n4 + ad; slot += kBlock) {
+        if (slot >= ad) store_stream<NT>(reinterpret_cast<f32x4 *>(dt) + (slot - ad), tile4[slot - ad]);
+      }
       for (uint32_t e = n4 * 4u + threadIdx.x; e < n; e += kBlock) dt[e] = tile[e];
       __syncthreads();
     }
