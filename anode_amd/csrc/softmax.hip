@@ -1321,11 +1321,14 @@ void launch_softmax_nd_typed(uint32_t P, uint32_t C, uint32_t N, const float *x,
 // the shape and on the sample number, and on nothing else.  All entry points (plain, with the label gather, with
 // the backward pass) run this kernel for these shapes, whatever the alignment of their arrays: their
 // probabilities agree to the bit.
-constexpr uint32_t kNdTileFloats = 4096;      // samples are gathered into tiles of 16 KB
-constexpr uint32_t kNdTileMaxSample = 8192;   // a larger sample has a tile to itself, up to 32 KB
-bool nd_tile_fits(uint32_t P, uint32_t C) {
-  return P > 1 && P < 1024 && P % 16u != 0 && C <= 64 && uint64_t(P) * C <= kNdTileMaxSample;
-}
+// Samples of more than 32 classes and up to 63 KB also have a tile to themselves where the planes are not whole
+// 32-byte pieces or too long for several threads per pixel ([196, 42] 3.8 -> 4.5 TB/s, [196, 70] 2.3 -> 3.4,
+// [100, 100] 2.7 -> 3.4; with few classes such samples are faster through the register kernels, [900, 12] 4.9
+// against 3.7, and short planes with several threads per pixel through the column tiles, [36, 128] 5.6 against 3.3).
+constexpr uint32_t kNdTileFloats = 4096;       // samples are gathered into tiles of 16 KB
+constexpr uint32_t kNdTileMaxSample = 8192;    // a larger sample has a tile to itself, up to 32 KB
+constexpr uint32_t kNdTileBigSample = 16128;   // ... and up to 63 KB from 33 classes on, where nothing else fits
+bool nd_tile_fits(uint32_t P, uint32_t C);
 
 template <bool NLL, bool BWD, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uint32_t C, uint32_t N, uint32_t SB,
@@ -1335,7 +1338,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
                                                                  float *__restrict__ nll,
                                                                  const float *__restrict__ dy,
                                                                  float *__restrict__ dx) {
-  extern __shared__ __align__(16) float tile[];  // SB * P * C floats, at most kNdTileMaxSample
+  extern __shared__ __align__(16) float tile[];  // SB * P * C floats, at most kNdTileBigSample
   f32x4 *tile4 = reinterpret_cast<f32x4 *>(tile);
   const uint32_t slab = P * C;
   for (uint64_t n0 = uint64_t(blockIdx.x) * SB; n0 < N; n0 += uint64_t(gridDim.x) * SB) {
@@ -1504,6 +1507,17 @@ ColTile nd_col_tile(uint32_t P, uint32_t C) {
   ct.tiles_per_sample = (P + TP - 1) / TP;
   ct.fits = true;
   return ct;
+}
+
+bool nd_tile_fits(uint32_t P, uint32_t C) {
+  if (!(P > 1 && P < 1024 && P % 16u != 0)) return false;
+  const uint64_t sample = uint64_t(P) * C;
+  if (C <= 64 && sample <= kNdTileMaxSample) return true;
+  if (C > 32 && sample <= kNdTileBigSample) {
+    const ColTile ct = nd_col_tile(P, C);
+    return !(ct.fits && ct.L >= 2);  // several threads per pixel over whole planes are faster
+  }
+  return false;
 }
 
 template <bool NLL, bool BWD, int NT>

@@ -196,7 +196,9 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
                                    (49, 20, 70), (7, 9, 1000), (4, 8, 4100), (2, 2, 9000), (512, 32, 3), (196, 64, 9),
                                    (9, 455, 6),
                                    # tiles of all classes of a run of pixels in LDS
-                                   (64, 300, 3), (196, 150, 2), (1028, 200, 1), (20, 70, 5), (16, 944, 1), (1056, 256, 2)])
+                                   (64, 300, 3), (196, 150, 2), (1028, 200, 1), (20, 70, 5), (16, 944, 1), (1056, 256, 2),
+                                   # samples of up to 63 KB with a tile to themselves
+                                   (196, 70, 3), (196, 82, 2), (100, 100, 2), (36, 128, 3)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

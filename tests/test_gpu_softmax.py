@@ -247,6 +247,9 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # (472, 944) and one more
              (64, 300, 3), (16, 900, 2), (16, 944, 1), (16, 945, 1), (784, 100, 2), (196, 150, 2), (2048, 472, 1),
              (2048, 473, 1), (20, 70, 5), (256, 65, 2), (1024, 193, 1), (1056, 200, 2), (1000, 65, 2),
+             # samples of up to 63 KB with a tile to themselves (more than 32 classes, planes that are not whole 64-byte
+             # pieces), the largest that fits and one class more, and a short plane that the column tiles keep
+             (196, 70, 3), (196, 82, 2), (196, 83, 2), (100, 100, 3), (36, 128, 3), (900, 17, 2), (252, 64, 2),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
