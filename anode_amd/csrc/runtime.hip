@@ -214,7 +214,11 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
       p.n_ctiles = ceil_div_u32(C, cb);
       const uint32_t gps = ceil_div_u32(uint64_t(cb) * S, vec ? 4u : 1u);  // 16-byte (or 4-byte) groups per sample
       p.J = kBlock / gps;
-      if (p.n_ctiles >= uint32_t(g_tuning.reduce_single_pass_grid)) {
+      // One tile per channel group where there are enough groups to fill the GPU, and also where a group's samples
+      // are few steps of the workgroup (at most 64: eight batches of loads): there the second launch costs more than
+      // the idle CUs lose ([784, 16, 32] batch_mean 9.6 -> 7.8 us, the nine batch-norm entry points 82 -> 65 us;
+      // [784, 16, 128], 128 steps, 12.0 us against 9.9 with sample tiles and the fold kernel).
+      if (p.n_ctiles >= uint32_t(g_tuning.reduce_single_pass_grid) || ceil_div_u32(N, p.J) <= 64u) {
         p.NB = N;  // one tile per channel group: no partial sums, no second kernel
       } else {
         uint64_t nb = per_tile / (uint64_t(cb) * S);
