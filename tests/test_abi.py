@@ -334,6 +334,20 @@ def test_reduction_tiling_on_drawn_shapes():
             _check_plan(dict(zip(keys, list(out))), S, C, N, bool(flags & 1))
 
 
+def test_lane_tiles_take_one_launch_for_few_steps_or_many_channel_groups():
+    # one partial per channel (no fold kernel, no scratch) where a channel group's samples are at most 64 steps of a
+    # workgroup, or where there are at least 256 channel groups; sample tiles and the fold kernel otherwise
+    def steps(p, N):
+        return -(-N // p["J"])
+    for S, C, N in [(784, 16, 32), (196, 32, 32), (49, 64, 32), (1024, 8, 64), (64, 128, 256), (49, 2048, 256)]:
+        p = _plan(S, C, N)
+        assert p["whole"] == 2 and (steps(p, N) <= 64 or p["n_ctiles"] >= 256), p
+        assert p["ppc"] == 1 and p["NB"] == N, p
+    for S, C, N in [(784, 16, 128), (784, 16, 4096), (196, 8, 100000)]:
+        p = _plan(S, C, N)
+        assert p["whole"] == 2 and steps(p, N) > 64 and p["n_ctiles"] < 256 and p["ppc"] > 1, p
+
+
 def test_reduction_tiling_without_lane_tiles():
     # tuning knob 9 = 0 switches lane tiles off: short channels then use the wide tiles (in a child process, so that
     # the knob does not leak into other tests)
