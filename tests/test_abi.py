@@ -346,6 +346,12 @@ def test_lane_tiles_take_one_launch_for_few_steps_or_many_channel_groups():
     for S, C, N in [(784, 16, 128), (784, 16, 4096), (196, 8, 100000)]:
         p = _plan(S, C, N)
         assert p["whole"] == 2 and steps(p, N) > 64 and p["n_ctiles"] < 256 and p["ppc"] > 1, p
+    # wide tiles (1024 < S <= 4096) up to 32 steps of 1024 positions (64 with at least 256 channel groups), chunk
+    # tiles (S > 4096) up to 56 steps of 1024 floats
+    for S, C, N, one in [(3136, 16, 8, True), (2048, 32, 16, True), (3136, 64, 16, False), (3136, 256, 16, True),
+                         (4096, 16, 16, False), (12544, 16, 4, True), (12544, 16, 5, False), (50176, 3, 1, False)]:
+        p = _plan(S, C, N)
+        assert p["whole"] in (0, 1) and (p["ppc"] == 1) == one, (S, C, N, p)
 
 
 def test_reduction_tiling_without_lane_tiles():
