@@ -97,6 +97,42 @@ def test_softmax_nd_beyond_2_31(big):
     del p, sums
 
 
+def test_softmax_nd_backward_beyond_2_31(big):
+    # planes of up to 131072 pixels: the backward pass walks the array flat, one 16-byte group of dx per thread
+    P, C, N = 1 << 16, 19, 1725
+    n = P * C * N
+    p = big[:n]                          # any values will do as "probabilities": the map is dy * (p - onehot)
+    lab = torch.randint(0, C + 1, (P * N,), device="cuda", dtype=torch.int32)   # C itself: out of range
+    dy = torch.randn(P * N, device="cuda")
+    dx = torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dy, p, lab, dx)
+    torch.cuda.synchronize()
+    pv, dv = p.view(N, C, P), dx.view(N, C, P)
+    ks = torch.arange(C, device="cuda", dtype=torch.int32).view(C, 1)
+    for i in (0, N // 2, N - 1):
+        want = dy.view(N, P)[i].unsqueeze(0) * (pv[i] - (lab.view(N, P)[i].unsqueeze(0) == ks).float())
+        assert torch.equal(dv[i], want), i
+    del dx
+
+
+def test_softmax_nd_many_classes_beyond_2_31(big):
+    # 220 classes: tiles of all classes of 32 pixels in LDS
+    P, C, N = 1 << 16, 220, 149          # 2 148 270 080 elements
+    n = P * C * N
+    assert (1 << 31) < n <= N_BIG
+    x = big[:n]
+    p = torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_packed_f32", P, C, N, x, p)
+    torch.cuda.synchronize()
+    pv = p.view(N, C, P)
+    for i in (0, N // 2, N - 1):
+        ref = torch.softmax(x.view(N, C, P)[i].double(), dim=0)
+        assert bool(((pv[i].double() - ref).abs() <= 1e-5 * ref).all())
+    sums = pv.sum(dim=1)
+    assert bool(((sums - 1).abs() < 1e-5).all())
+    del p, sums
+
+
 def test_short_channels_beyond_2_31(big):
     # 7x7 maps: the reductions run as lane tiles (one launch, all samples per workgroup), the maps walk channels of
     # 49 elements; sample offsets n * C * S pass 2^31
@@ -152,6 +188,31 @@ def test_row_softmax_head_beyond_2_31(big):
         assert torch.equal(dv[rows], 0.5 * (pv[rows] - onehot))
         top = torch.gather(xv[rows], 1, idx[rows].long().unsqueeze(1)).squeeze(1)
         assert torch.equal(top, xv[rows].max(dim=1).values)
+    sums = pv.sum(dim=1)
+    assert bool(((sums - 1).abs() < 1e-5).all())
+    del p, dx, sums
+
+
+def test_long_odd_rows_beyond_2_31(big):
+    # rows of 50 257 classes start anywhere in a 16-byte group: the streaming kernel over the array's aligned groups
+    K, R = 50257, 42750                  # 2 148 486 750 elements
+    n = K * R
+    assert (1 << 31) < n <= N_BIG
+    x = big[:n]
+    lab = torch.randint(0, K, (R,), device="cuda", dtype=torch.int32)
+    dy = torch.full((R,), 0.25, device="cuda")
+    p, nll, dx = torch.empty(n, device="cuda"), torch.empty(R, device="cuda"), torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32", K, R, x, lab, dy, p, nll, dx)
+    torch.cuda.synchronize()
+    pv, xv, dv = p.view(R, K), x.view(R, K), dx.view(R, K)
+    for lo in (0, (1 << 31) // K - 10, R - 20):        # the first rows, rows across 2^31, the last rows
+        rows = slice(lo, lo + 20)
+        ref = torch.softmax(xv[rows].double(), dim=1)
+        assert bool(((pv[rows].double() - ref).abs() <= 1e-5 * ref).all())
+        picked = torch.gather(pv[rows], 1, lab[rows].long().unsqueeze(1)).squeeze(1)
+        assert torch.allclose(nll[rows], -torch.log(picked), rtol=1e-5, atol=1e-6)
+        onehot = torch.nn.functional.one_hot(lab[rows].long(), K).float()
+        assert torch.equal(dv[rows], 0.25 * (pv[rows] - onehot))
     sums = pv.sum(dim=1)
     assert bool(((sums - 1).abs() < 1e-5).all())
     del p, dx, sums
