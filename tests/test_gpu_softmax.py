@@ -56,6 +56,8 @@ ROW_SHAPES = [(1, 5), (2, 7), (3, 1000), (10, 32), (19, 513), (32, 2), (33, 9), 
               (180, 41), (215, 37),
               # rows in registers that start at every distance from a 128-byte line (K = 4 * odd)
               (212, 40), (1012, 19), (2044, 9), (2052, 11), (4100, 9), (8196, 3),
+              # few rows of 513 to 2048 classes: a workgroup per row (16-byte accesses), and its neighbours
+              (516, 7), (1000, 256), (1024, 512), (1028, 512), (2048, 40), (1000, 513), (512, 7),
               # the limits of the workgroup-per-row register kernel
               (4096, 3), (4097, 2), (8192, 2), (8193, 1), (16384, 2), (16385, 1),
               # ... and of its 512-thread form (rows of 9217 to 16384 classes)
