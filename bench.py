@@ -67,9 +67,9 @@ MEASURED_TRAFFIC = {
     ("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", "bn_bwd_cfg2b"): 205583995,
     ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): 308430450,
     ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): 1610539015,
-    ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): 637595130,
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): 291278293,
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): 671289838,
+    ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): 637591035,
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): 291192285,
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): 671287790,
     ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): 192705077,
     ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): 192703030,
 }
