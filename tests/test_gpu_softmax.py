@@ -291,6 +291,46 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
         assert_bit_exact(host(dxa), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab, dx_in=old), "nd bwd acc vs fp32")
 
 
+@pytest.mark.parametrize("P,C,N", [(64, 19, 3), (196, 19, 5), (196, 70, 3), (64, 300, 2), (1056, 200, 1), (2048, 19, 2),
+                                   (1028, 300, 1), (36, 128, 3)])
+def test_softmax_nd_arrays_that_lie_differently(oracle, P, C, N):
+    # every n-d kernel family with arrays at different element offsets from a 16-byte boundary: the 16-byte forms
+    # need all of a launch's arrays aligned, and any mix must still give the 4-byte forms' (correct) results;
+    # the plain and the fused entry points, and guard bands round the outputs
+    import torch
+    g = np.random.default_rng(P + 7 * C)
+    n = P * C * N
+    x = g.standard_normal(n).astype(F32)
+    lab = g.integers(0, C, P * N).astype(np.uint32)
+    dy = g.standard_normal(P * N).astype(F32)
+    want = oracle.softmax_nd(P, C, N, x, f64=True)
+
+    def guarded(count, off, fill):
+        buf = torch.full((count + 40,), fill, dtype=torch.float32, device="cuda")
+        return buf, buf[16 + off:16 + off + count]
+
+    def intact(buf, count, off, fill):
+        h = host(buf)
+        return bool(np.all(h[:16 + off] == fill) and np.all(h[16 + off + count:] == fill))
+
+    for off_x, off_y, off_dx, off_lab in [(0, 0, 0, 0), (0, 1, 0, 0), (1, 0, 0, 0), (0, 0, 2, 0), (0, 0, 0, 1), (3, 2, 1, 3)]:
+        print(f"case P={P} C={C} N={N} offsets {off_x} {off_y} {off_dx} {off_lab}", flush=True)
+        ybuf, y = guarded(n, off_y, 777.0)
+        call("anode_gpu_softmax_nd_packed_f32", P, C, N, dev(x, off_x), y)
+        assert intact(ybuf, n, off_y, 777.0)
+        assert_close(host(y), want, "softmax_nd", abs_floor=1e-30)
+        y2buf, y2 = guarded(n, off_y, 777.0)
+        dbuf, dx = guarded(n, off_dx, 555.0)
+        nbuf, nll = guarded(P * N, off_lab, 333.0)
+        call("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", P, C, N, dev(x, off_x), dev(lab, off_lab),
+             dev(dy, off_lab), y2, nll, dx)
+        assert intact(y2buf, n, off_y, 777.0) and intact(dbuf, n, off_dx, 555.0) and intact(nbuf, P * N, off_lab, 333.0)
+        p = host(y2)
+        assert_close(p, want, "fused softmax_nd", abs_floor=1e-30)
+        assert_close(host(nll), oracle.softmax_nd_cat_nll(P, C, N, p, lab, f64=True), "fused nll", abs_floor=1e-6)
+        assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "fused dx vs fp32 of its own p")
+
+
 @pytest.mark.parametrize("P", [8, 1028])
 @pytest.mark.parametrize("C", [3, 19, 40, 100, 200, 300])
 def test_softmax_nd_special_values(oracle, C, P):
