@@ -148,14 +148,17 @@ def test_softmax_long_rows_special_values(oracle, K):
 
 
 @pytest.mark.parametrize("K,R", [(32773, 5), (50257, 3), (40002, 4), (65536, 3),
+                                 # shorter rows: every row kernel family with arrays that lie differently
+                                 (10, 3000), (33, 700), (100, 300), (250, 100), (1000, 256), (1001, 30), (2048, 12),
                                  # rows in registers: every workgroup size, and the longest row that fits each
                                  (2050, 5), (4062, 3), (4063, 3), (8158, 2), (8159, 2), (12289, 3), (16350, 2), (16351, 2),
                                  (30522, 2), (32734, 2), (32735, 2)])
-def test_softmax_long_rows_touch_nothing_but_their_rows(oracle, K, R):
-    # Rows of more than 2048 classes that do not start on 16-byte boundaries are read and written in the array's 16-byte groups where x
-    # and y start equally far from such a boundary: the groups at a row's ends are shared with its neighbours, and
-    # with whatever lies before and after the array.  Guard bands around y must come back untouched, for every
-    # distance from a boundary, and also where x and y lie differently (4-byte accesses).
+def test_softmax_rows_touch_nothing_but_their_rows(oracle, K, R):
+    # Rows of more than 32768 classes that do not start on 16-byte boundaries are read and written in the array's
+    # 16-byte groups where x and y start equally far from such a boundary: the groups at a row's ends are shared with
+    # its neighbours, and with whatever lies before and after the array.  Guard bands around y (and dx) must come
+    # back untouched, for every distance from a boundary, and also where x and y lie differently (4-byte accesses);
+    # the same for the kernels of shorter rows, whose 16-byte forms need every array of the launch aligned.
     import torch
     g = np.random.default_rng(K + R)
     x = (2 * g.standard_normal(K * R)).astype(F32)
