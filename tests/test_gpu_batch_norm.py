@@ -191,3 +191,52 @@ def test_batch_norm_on_a_side_stream(oracle):
     m0 = empty(C)
     call("anode_gpu_batch_mean_3d1_packed_f32", S, C, N, xd, m0, stream=0)
     assert_bit_exact(host(m0), host(m), "null stream")
+
+
+@pytest.mark.parametrize("S,C,N", [(784, 16, 8), (49, 40, 16), (3136, 4, 3), (12544, 3, 2), (4, 64, 50), (1, 300, 40)])
+def test_batch_norm_arrays_that_lie_differently(oracle, S, C, N):
+    # the 16-byte forms need every array of a launch on a 16-byte boundary; with any mix of element offsets the
+    # element-wide forms must give the same results, and nothing outside the outputs may be written
+    import torch
+    eps = 1e-5
+    x, dy = make(S, C, N, seed=S + 13 * C)
+    n = x.size
+    dims = (S, C, N)
+    mean = oracle.batch_mean(*dims, x)
+    var = oracle.batch_var(*dims, eps, x, mean)
+    dvar = np.random.default_rng(3).standard_normal(C).astype(F32)
+    old = np.random.default_rng(4).standard_normal(n).astype(F32)
+
+    def guarded(values_or_count, off, fill=4242.0):
+        count = values_or_count if isinstance(values_or_count, int) else values_or_count.size
+        buf = torch.full((count + 40,), fill, dtype=torch.float32, device="cuda")
+        view = buf[16 + off:16 + off + count]
+        if not isinstance(values_or_count, int):
+            view.copy_(torch.from_numpy(values_or_count))
+        return buf, view
+
+    def intact(buf, count, off, fill=4242.0):
+        h = host(buf)
+        return bool(np.all(h[:16 + off] == fill) and np.all(h[16 + off + count:] == fill))
+
+    for off_x, off_dy, off_out in [(0, 0, 1), (1, 0, 0), (0, 2, 0), (3, 1, 2), (2, 2, 0)]:
+        print(f"case S={S} C={C} N={N} offsets {off_x} {off_dy} {off_out}", flush=True)
+        xd, dyd = dev(x, off_x), dev(dy, off_dy)
+        md, vd = dev(mean, off_dy), dev(var, off_x)
+        ybuf, y = guarded(n, off_out)
+        call("anode_gpu_batch_norm_3d1_packed_f32", *dims, xd, md, vd, y)
+        assert intact(ybuf, n, off_out)
+        assert_bit_exact(host(y), oracle.batch_norm(*dims, x, mean, var), "norm")
+        abuf, acc = guarded(old, off_out)
+        call("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", *dims, dev(dvar, off_out), xd, md, acc)
+        assert intact(abuf, n, off_out)
+        assert_bit_exact(host(acc), oracle.batch_var_bwd(*dims, dvar, x, mean, dx_in=old), "var_bwd accumulate")
+        cbuf, out = guarded(C, off_out)
+        call("anode_gpu_batch_mean_3d1_packed_f32", *dims, xd, out)
+        assert intact(cbuf, C, off_out)
+        assert_close(host(out), oracle.batch_mean(*dims, x, f64=True), "mean")
+        cbuf, out = guarded(C, off_out)
+        call("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", *dims, dyd, xd, md, vd, out)
+        assert intact(cbuf, C, off_out)
+        ref = oracle.batch_norm_bwd_var(*dims, dy, x, mean, var, f64=True)
+        assert_close(host(out), ref, "norm_bwd_var", abs_floor=1e-6 * rms(ref))
