@@ -93,6 +93,30 @@ def test_two_input_maps_and_in_place_backward(oracle):
             assert_bit_exact(host(buf), oracle.flat_map2("positive_clip_bwd", a, b), "in-place relu bwd")
 
 
+def test_maps_with_arrays_that_lie_differently(oracle):
+    # one- and two-input maps with every array at its own element offset, guard bands round the output
+    import torch
+    for n in (7, 1027, 300001):
+        a, b = data(n, 6), data(n, 7)[::-1].copy()
+        for off_a, off_b, off_out in [(0, 0, 1), (1, 0, 0), (0, 3, 0), (1, 2, 3), (2, 2, 0)]:
+            for name, op, two in [("anode_gpu_positive_clip_flat_map_bwd_f32", "positive_clip_bwd", True),
+                                  ("anode_gpu_M1_copy_map_M2_unit_step_map_R_product_reduce_flat_join_f32",
+                                   "copy_unit_step_join", True),
+                                  ("anode_gpu_square_flat_map_f32", "square", False)]:
+                buf = torch.full((n + 40,), 9191.0, dtype=torch.float32, device="cuda")
+                out = buf[16 + off_out:16 + off_out + n]
+                if two:
+                    call(name, n, dev(a, off_a), dev(b, off_b), out)
+                    want = oracle.flat_map2(op, a, b)
+                else:
+                    call(name, n, dev(a, off_a), out)
+                    want = oracle.flat_map(op, a)
+                h = host(buf)
+                assert np.all(h[:16 + off_out] == 9191.0) and np.all(h[16 + off_out + n:] == 9191.0), (name, n)
+                with np.errstate(all="ignore"):
+                    assert_bit_exact(h[16 + off_out:16 + off_out + n], want, f"{op} n={n} offsets {off_a} {off_b} {off_out}")
+
+
 @pytest.mark.parametrize("c", [0.01, 0.0, -0.5, 2.0])
 def test_leaky_relu(oracle, c):
     n = 70001
