@@ -645,7 +645,9 @@ ANODE_EXPORT int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, 
                                                                  float epsilon, const float *x, float *mean,
                                                                  float *var, const KernelConfig *,
                                                                  CUstream_st *stream) {
-  // Sizes are checked before anything touches the device, so that a refusal has no side effect.
+  // Sizes are checked before anything touches the device, so that a refusal has no side effect; the element count
+  // first, as in every other entry point (the tiling below is not planned for counts that do not fit 32 bits).
+  (void)checked_len(dim0, dim1, dim2, __func__);
   const bool ptrs_aligned = aligned16(x);
   const ReducePlan pl = plan_chan_reduce(dim0, dim1, dim2, ptrs_aligned, uint32_t(tuning().reduce_wg_target),
                                          MeanVarReduce::NIN);

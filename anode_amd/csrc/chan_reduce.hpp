@@ -513,7 +513,7 @@ int launch_chan_reduce(const char *symbol, uint32_t S, uint32_t C, uint32_t N, O
   if (Op::NIN < 3) c = a;
   const int nt = stream_policy(size_t(len) * sizeof(float), tuning().reduce_nontemporal);
 
-  ScratchLease lease{nullptr, std::unique_lock<std::mutex>()};
+  ScratchLease lease{nullptr, std::unique_lock<std::mutex>(), nullptr};
   double *part = nullptr;
   const size_t need = chan_reduce_scratch_bytes(pl, Op::NACC);
   if (need > 0) {

@@ -8,6 +8,7 @@
 #include <atomic>
 #include <cstddef>
 #include <cstdint>
+#include <memory>
 #include <mutex>
 #include <type_traits>
 
@@ -272,15 +273,17 @@ void note_launch(const char *symbol);
 void note_error(const char *symbol, hipError_t e, const char *what);
 
 // A device buffer private to (current device, stream), grown on demand and
-// kept until anode_gpu_release_scratch().  The lease holds the cache's lock: keep it
-// alive until every kernel that uses the buffer has been enqueued, so that two
-// host threads sharing a stream cannot interleave their launches.  When the
-// buffer cannot be provided (allocation failure, or the stream is being captured
-// and would have to allocate) the error is recorded under `symbol`, ptr is null
-// and the lock is not held: the caller skips its launch.
+// kept until anode_gpu_release_scratch().  The lease holds that buffer's own lock
+// (not a lock of the whole cache): keep it alive until every kernel that uses the
+// buffer has been enqueued, so that two host threads sharing a stream cannot
+// interleave their launches; threads on other streams or devices are not held up.
+// When the buffer cannot be provided (allocation failure, or the stream is being
+// captured and would have to allocate) the error is recorded under `symbol`, ptr
+// is null and the lock is not held: the caller skips its launch.
 struct ScratchLease {
   void *ptr;
   std::unique_lock<std::mutex> lock;
+  std::shared_ptr<void> owner;  // keeps the cache entry (and with it the mutex) alive while the lease is
 };
 ScratchLease acquire_scratch(hipStream_t stream, size_t bytes, const char *symbol);
 

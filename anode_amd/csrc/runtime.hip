@@ -8,6 +8,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <memory>
+#include <mutex>
 #include <utility>
 #include <vector>
 
@@ -19,13 +21,19 @@ constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
 std::atomic<int> g_last_error{0};
 
+// One buffer per (device, stream), each behind a lock of its own: a reduction holds its stream's lock from the
+// lookup until both of its kernels are enqueued, so host threads that share a stream cannot interleave their
+// launches, while threads on different streams or devices never wait for each other.  The map's own lock is held
+// for the lookup only.  Entries are shared_ptrs: anode_gpu_release_scratch() takes an entry out of the map and
+// frees its buffers once no lease holds it.
 struct ScratchBuf {
+  std::mutex mu;
   void *ptr = nullptr;
   size_t cap = 0;
   std::vector<void *> outgrown;  // earlier, smaller buffers: kernels in flight may still use them
 };
-std::mutex g_scratch_mutex;
-std::map<std::pair<int, hipStream_t>, ScratchBuf> g_scratch;
+std::mutex g_scratch_map_mutex;
+std::map<std::pair<int, hipStream_t>, std::shared_ptr<ScratchBuf>> g_scratch;
 
 Tuning g_tuning = {
     /*flat_wg_per_cu=*/{{0}},
@@ -294,15 +302,30 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
 }
 
 ScratchLease acquire_scratch(hipStream_t stream, size_t bytes, const char *symbol) {
-  ScratchLease lease{nullptr, std::unique_lock<std::mutex>(g_scratch_mutex)};
   int dev = 0;
   (void)hipGetDevice(&dev);
-  ScratchBuf &buf = g_scratch[std::make_pair(dev, stream)];
+  std::shared_ptr<ScratchBuf> entry;
+  {
+    std::lock_guard<std::mutex> map_lock(g_scratch_map_mutex);
+    std::shared_ptr<ScratchBuf> &slot = g_scratch[std::make_pair(dev, stream)];
+    if (!slot) slot = std::make_shared<ScratchBuf>();
+    entry = slot;
+  }
+  ScratchLease lease{nullptr, std::unique_lock<std::mutex>(entry->mu), entry};
+  ScratchBuf &buf = *entry;
   if (buf.cap < bytes) {
     // Growing means hipMalloc, which a stream under capture cannot take (it would fail and could invalidate the
-    // capture): refuse instead, and tell the caller how to avoid it.
+    // capture): refuse instead, and tell the caller how to avoid it.  A query that itself fails (no device; the
+    // legacy stream while another stream is being captured in global mode) refuses as well: nothing is allocated
+    // on a stream whose state is unknown.
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone) {
+    const hipError_t q = hipStreamIsCapturing(stream, &capturing);
+    if (q != hipSuccess) {
+      note_error(symbol, q, "cannot read the capture state of the stream, so the reduction scratch is not allocated");
+      lease.lock.unlock();
+      return lease;
+    }
+    if (capturing != hipStreamCaptureStatusNone) {
       note_error(symbol, hipErrorStreamCaptureUnsupported,
                  "the stream is being captured and has no reduction scratch yet (call anode_gpu_reserve_scratch "
                  "or run the entry point once on this stream before capturing)");
@@ -363,15 +386,24 @@ ANODE_EXPORT int anode_gpu_reserve_scratch(CUstream_st *stream, size_t bytes) {
 // Frees every scratch buffer held for `stream` on the current device.  The caller must have synchronised the
 // stream: kernels in flight would lose their partial sums.  Returns the number of buffers freed.
 ANODE_EXPORT int anode_gpu_release_scratch(CUstream_st *stream) {
-  std::lock_guard<std::mutex> lock(anode::g_scratch_mutex);
   int dev = 0;
   (void)hipGetDevice(&dev);
-  const auto it = anode::g_scratch.find(std::make_pair(dev, anode::as_stream(stream)));
-  if (it == anode::g_scratch.end()) return 0;
+  std::shared_ptr<anode::ScratchBuf> entry;
+  {
+    std::lock_guard<std::mutex> map_lock(anode::g_scratch_map_mutex);
+    const auto it = anode::g_scratch.find(std::make_pair(dev, anode::as_stream(stream)));
+    if (it == anode::g_scratch.end()) return 0;
+    entry = it->second;
+    anode::g_scratch.erase(it);
+  }
+  if (!entry) return 0;
+  std::lock_guard<std::mutex> lock(entry->mu);  // a call that is still enqueueing on this stream finishes first
   int freed = 0;
-  for (void *p : it->second.outgrown) freed += (hipFree(p) == hipSuccess);
-  if (it->second.ptr) freed += (hipFree(it->second.ptr) == hipSuccess);
-  anode::g_scratch.erase(it);
+  for (void *p : entry->outgrown) freed += (hipFree(p) == hipSuccess);
+  if (entry->ptr) freed += (hipFree(entry->ptr) == hipSuccess);
+  entry->outgrown.clear();
+  entry->ptr = nullptr;
+  entry->cap = 0;
   return freed;
 }
 

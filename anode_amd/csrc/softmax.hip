@@ -1363,8 +1363,10 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
     // A wave's step covers whole 128-byte lines of the array: the groups are taken `ax` places later, ax = the
     // tile's distance in groups from the line before it, so that the first wave's first step is the short one
     // (a sample of 19 planes of 196 pixels starts anywhere in a line; [196, 19] 4.9 -> 5.2 TB/s, [49, 19] 4.8 -> 5.3).
+    // (a tile of fewer than four floats -- a last tile of one sample of a 2- or 3-pixel, one-class array -- has no
+    // group to clamp to: it takes the element loop below alone)
     const uint32_t ax = vec ? uint32_t((reinterpret_cast<uintptr_t>(xt) >> 4) & 7u) : 0u;
-    for (uint32_t g0 = 0; g0 < n4 + ax; g0 += 8u * kBlock) {
+    for (uint32_t g0 = 0; n4 != 0u && g0 < n4 + ax; g0 += 8u * kBlock) {
       f32x4 in[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -1684,6 +1686,9 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
 // exponentials are added, hence the bits of p, depends on the kernel.
 bool nd_one_pixel_per_thread(uint32_t P, uint32_t C, bool vec) { return (!vec || P < 1024) && C > 32 && C <= 128; }
 
+// whether the plain n-d entry point takes its 16-byte kernels: decided by the plane length and by x and y alone
+bool nd_vec_xy(uint32_t P, const float *x, const float *y) { return (P % 4 == 0) && aligned16(x) && aligned16(y); }
+
 void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                        CUstream_st *stream) {
   const uint32_t len = checked_len(P, C, N, symbol);
@@ -1693,7 +1698,7 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     return;
   }
   hipStream_t s = as_stream(stream);
-  const bool vec = (P % 4 == 0) && aligned16(x) && aligned16(y);
+  const bool vec = nd_vec_xy(P, x, y);
   const ColTile ct = nd_col_tile(P, C);
   if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
@@ -1938,7 +1943,11 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll);
-             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
+             // the kernel family (and with it the order of a pixel's sum) follows x and softmax alone, as in the
+             // plain entry point: where those two allow 16-byte accesses and the label or nll array does not, the
+             // two passes run back to back instead of a kernel that would round differently
+             vec == nd_vec_xy(prefix_dim, x, softmax) &&
+             (dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec)))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
@@ -1976,7 +1985,9 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
     note_launch(__func__);
   } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
                               aligned16(nll) && aligned16(dy) && aligned16(dx);
-             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
+             // (as above: a label, nll, dy or dx array that lies differently sends the call to the three passes)
+             vec == nd_vec_xy(prefix_dim, x, softmax) &&
+             (dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec)))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);

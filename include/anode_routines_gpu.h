@@ -328,7 +328,10 @@ size_t anode_host_arg_max_f32(const float *xs, size_t len);
  * hipError_t for anode_gpu_take_last_error().  A HIP graph keeps the buffer of the stream it was captured on: graphs
  * captured on one stream must not be replayed concurrently with each other or with eager reduction calls on that
  * stream. */
-/* Upper bound of the scratch bytes any reduction entry point needs for a [dim0, dim1, dim2] array. */
+/* Upper bound of the scratch bytes any reduction entry point needs for a [dim0, dim1, dim2] array, for either
+ * alignment of its arrays.  The bound holds for the library's tiling as it is when the function is called: the
+ * tiling is fixed for a build and only moves through the library's undeclared measurement hook, after which the
+ * query must be repeated. */
 size_t anode_gpu_reduce_scratch_bytes(uint32_t dim0, uint32_t dim1, uint32_t dim2);
 /* Makes `stream` (current device) hold at least `bytes` of scratch, so that later calls allocate nothing (call it
  * before capturing the stream).  Returns 0 or the hipError_t of the failed allocation. */
@@ -339,7 +342,11 @@ int anode_gpu_release_scratch(struct CUstream_st *stream);
 
 /* Library introspection.  No reference counterpart. */
 /* 0 when no launch made by this library has failed since the last call; otherwise the hipError_t
- * of the most recent failure.  Reading clears it (the thread's own HIP error state is never cleared by this library). */
+ * of the most recent failure.  Reading clears it.  The thread's own HIP error state is never cleared by this library
+ * (the reference's kernels leave it to the caller, whose own checks must keep seeing what they see today): a failed
+ * launch is noticed by peeking at that state, so while the caller leaves an error pending there (no
+ * hipGetLastError()), a later launch that fails with the same hipError_t cannot be told from the pending one and is
+ * not recorded again.  Refusals (scratch unavailable, stream under capture) are always recorded. */
 int anode_gpu_take_last_error(void);
 /* Number of entry points of Part 1 (46). */
 uint32_t anode_gpu_reference_symbol_count(void);

@@ -216,7 +216,9 @@ def test_scratch_allocation_failure_is_reported_not_fatal():
     assert err != 0 and again == 0
     assert out["noalloc"] == ["1", "0"]                  # refused by size: not a HIP error
     assert out["released"] == ["0"] and "alive" in out
-    assert "cannot allocate the reduction scratch" in r.stderr and "nothing was enqueued" in r.stderr
+    # (without a device even the stream's capture state cannot be read: refused at that point, before any allocation)
+    assert ("cannot allocate the reduction scratch" in r.stderr or "the reduction scratch is not allocated" in r.stderr)
+    assert "nothing was enqueued" in r.stderr
     assert "anode_gpu_batch_mean_3d1_packed_f32" in r.stderr
     assert "more than the 4194304 bytes of the static scratch array" in r.stderr
 

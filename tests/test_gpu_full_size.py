@@ -38,6 +38,43 @@ def test_config1_u8_image_batch_cast_and_dequantize(oracle):
     assert_bit_exact(host(u).view(np.uint32), oracle.upcast_u8(q), "upcast 38.5M")
 
 
+def test_config1_additive_full_size(oracle):
+    """What config 1 words beyond the reference's two casts, at [256,3,224,224]: u8 -> f32 with per-channel
+    ImageNet normalisation in one pass, and an N(0,1) f32 tensor quantised to u8 (scale 8/255, zero point at -4,
+    round-half-even).  Bit-exact against the oracle; the quantiser has no counterpart in the reference."""
+    n_img, C, S = 256, 3, 224 * 224
+    n = n_img * C * S
+    g = np.random.default_rng(1)
+    q = g.integers(0, 256, n, dtype=np.uint8)
+    mean = np.array([0.485, 0.456, 0.406], F32)
+    std = np.array([0.229, 0.224, 0.225], F32)
+    a = (F32(1.0) / (F32(255.0) * std)).astype(F32)
+    b = (-mean / std).astype(F32)
+    y = empty(n)
+    call("anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32", S, C, n_img, dev(a), dev(b), dev(q), y)
+    yh = host(y)
+    assert_bit_exact(yh, oracle.bcast_dequantize_u8(S, C, n_img, a, b, q), "per-channel dequantize 38.5M")
+    # size-independent: undoing the affine per channel recovers every code
+    ch = np.tile(np.repeat(np.arange(C), S), n_img)
+    back = np.rint((yh.astype(np.float64) - b.astype(np.float64)[ch]) / a.astype(np.float64)[ch])
+    assert np.array_equal(back.astype(np.uint8), q)
+    del yh, back, ch
+
+    z = g.standard_normal(n, dtype=np.float32)
+    zq = empty(n, dtype=torch.uint8)
+    call("anode_gpu_quantize_u8_packed_f32", n, -4.0, 4.0, dev(z), zq)
+    zh = host(zq)
+    assert_bit_exact(zh, oracle.quantize_u8(-4.0, 4.0, z), "quantize 38.5M")
+    # dequantising the codes lands within half a step of the clamped input, and quantising again is the identity
+    deq = empty(n)
+    call("anode_gpu_dequantize_u8_packed_f32", n, -4.0, 4.0, zq, deq)
+    step = 8.0 / 255.0
+    assert float(np.max(np.abs(host(deq).astype(np.float64) - np.clip(z, -4, 4)))) <= 0.5 * step * (1 + 1e-5)
+    zq2 = empty(n, dtype=torch.uint8)
+    call("anode_gpu_quantize_u8_packed_f32", n, -4.0, 4.0, deq, zq2)
+    assert np.array_equal(host(zq2), zh)
+
+
 def _bn_full(oracle, S, C, N, seed, mean_shift, std, slice_samples):
     """BN forward + backward launch set at full size."""
     eps = 1e-5

@@ -330,8 +330,48 @@ def test_softmax_nd_arrays_that_lie_differently(oracle, P, C, N):
         assert intact(y2buf, n, off_y, 777.0) and intact(dbuf, n, off_dx, 555.0) and intact(nbuf, P * N, off_lab, 333.0)
         p = host(y2)
         assert_close(p, want, "fused softmax_nd", abs_floor=1e-30)
+        assert_bit_exact(p, host(y), "fused p vs plain p, whatever the label / nll / dy / dx arrays' alignment")
         assert_close(host(nll), oracle.softmax_nd_cat_nll(P, C, N, p, lab, f64=True), "fused nll", abs_floor=1e-6)
         assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "fused dx vs fp32 of its own p")
+
+
+@pytest.mark.parametrize("P,C,N,off", [(2, 1, 2053, 0), (3, 1, 1, 4), (2, 1, 1, 4), (3, 1, 2049, 0), (2, 1, 2053, 4),
+                                       (1, 3, 1, 4), (1, 2, 4097, 0)])
+def test_softmax_nd_tile_of_fewer_than_four_floats(oracle, P, C, N, off):
+    # the LDS-tile kernel with a last tile (or an only tile) of fewer than four floats that does not start on a
+    # 128-byte line: it has no 16-byte group of its own and must go through the element loop alone.  The arrays lie
+    # `off` floats into their allocations (16-byte aligned either way), with guard bands; plain and fused entry points.
+    import torch
+    g = np.random.default_rng(P + 5 * N)
+    n = P * C * N
+    x = g.standard_normal(n).astype(F32)
+    lab = g.integers(0, C, P * N).astype(np.uint32)
+    dy = g.standard_normal(P * N).astype(F32)
+    want = oracle.softmax_nd(P, C, N, x, f64=True)
+
+    def guarded(count, fill):
+        buf = torch.full((count + 64,), fill, dtype=torch.float32, device="cuda")
+        return buf, buf[32 + off:32 + off + count]
+
+    def intact(buf, count, fill):
+        h = host(buf)
+        return bool(np.all(h[:32 + off] == fill) and np.all(h[32 + off + count:] == fill))
+
+    xbuf, xd = guarded(n, 0.0)
+    xd.copy_(torch.from_numpy(x))
+    ybuf, y = guarded(n, 777.0)
+    call("anode_gpu_softmax_nd_packed_f32", P, C, N, xd, y)
+    assert intact(ybuf, n, 777.0)
+    assert_close(host(y), want, "softmax_nd", abs_floor=1e-30)
+    y2buf, y2 = guarded(n, 777.0)
+    dbuf, dx = guarded(n, 555.0)
+    nbuf, nll = guarded(P * N, 333.0)
+    call("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", P, C, N, xd, dev(lab), dev(dy), y2, nll, dx)
+    assert intact(y2buf, n, 777.0) and intact(dbuf, n, 555.0) and intact(nbuf, P * N, 333.0)
+    p = host(y2)
+    assert_bit_exact(p, host(y), "fused p vs plain p")
+    assert_close(host(nll), oracle.softmax_nd_cat_nll(P, C, N, p, lab, f64=True), "fused nll", abs_floor=1e-6)
+    assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "fused dx vs fp32 of its own p")
 
 
 @pytest.mark.parametrize("P", [8, 1028])

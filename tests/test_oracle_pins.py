@@ -555,3 +555,136 @@ def test_bcast_affine_and_mean_var(oracle):
     xt = torch.from_numpy(x).double()
     np.testing.assert_allclose(m, xt.mean((0, 2, 3)).numpy(), rtol=1e-13)
     np.testing.assert_allclose(v, xt.var((0, 2, 3), unbiased=False).numpy() + float(F32(1e-5)), rtol=1e-12)
+
+
+# --------------------------------------------------------------------------
+# the additive reductions / maps and the gpudevicemem neighbours
+# --------------------------------------------------------------------------
+
+def test_channel_sum_triple_loop_on_a_lopsided_array(oracle):
+    # the commented-out declarations lib.h:408-430: y[b] = sum over a and c of x[a,b,c] (or of its square).
+    # All three extents differ, so a transposed extent or a sum over the wrong axis lands on other numbers.
+    d0, d1, d2 = 5, 3, 2
+    x = (rng(41).standard_normal(d0 * d1 * d2) * 3 + 1).astype(F32)
+    plain = [0.0] * d1
+    squares = [0.0] * d1
+    for c in range(d2):
+        for b in range(d1):
+            for a in range(d0):
+                v = float(x[a + d0 * (b + d1 * c)])
+                plain[b] += v
+                squares[b] += v * v
+    np.testing.assert_allclose(oracle.channel_sum(d0, d1, d2, x), plain, rtol=1e-14)
+    np.testing.assert_allclose(oracle.channel_sum(d0, d1, d2, x, square=True), squares, rtol=1e-14)
+    assert not np.allclose(plain, squares)
+    # integers: the sums are exact, whatever the order
+    xi = np.arange(d0 * d1 * d2, dtype=F32)
+    t = xi.reshape(d2, d1, d0).astype(np.float64)
+    assert np.array_equal(oracle.channel_sum(d0, d1, d2, xi), t.sum((0, 2)))
+    assert np.array_equal(oracle.channel_sum(d0, d1, d2, xi, square=True), (t * t).sum((0, 2)))
+    # against torch float64 on an NCHW view
+    xt = torch.from_numpy(x.reshape(d2, d1, d0)).double()
+    np.testing.assert_allclose(oracle.channel_sum(d0, d1, d2, x), xt.sum((0, 2)).numpy(), rtol=1e-14)
+
+
+def test_batch_norm_affine_is_one_fma_over_the_pinned_batch_norm(oracle):
+    # y = fma(batch_norm(x)[c], gamma[c], beta[c]): composed from batch_norm (pinned against torch float64 above)
+    # with exact rational arithmetic for the one rounding, and against torch's own affine batch norm.
+    N, C, H, W = 3, 4, 2, 5
+    S = H * W
+    g = rng(42)
+    x = (2 + 3 * g.standard_normal((N, C, H, W))).astype(F32)
+    gamma = g.uniform(0.5, 1.5, C).astype(F32)
+    beta = (0.1 * g.standard_normal(C)).astype(F32)
+    eps = F32(1e-5)
+    xf = nchw_to_flat(x)
+    mean = oracle.batch_mean(S, C, N, xf)
+    var = oracle.batch_var(S, C, N, eps, xf, mean)
+    yn = oracle.batch_norm(S, C, N, xf, mean, var)
+    got = oracle.batch_norm_affine(S, C, N, xf, mean, var, gamma, beta)
+    assert got.dtype == F32
+    want = np.empty_like(got)
+    for i in range(got.size):
+        c = (i // S) % C
+        want[i] = _round_fraction_to_f32(Fraction(float(yn[i])) * Fraction(float(gamma[c])) + Fraction(float(beta[c])))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # an unfused multiply-then-add differs somewhere, so the pin above can fail
+    unfused = (yn * gamma[(np.arange(got.size) // S) % C] + beta[(np.arange(got.size) // S) % C]).astype(F32)
+    assert np.any(unfused != got)
+    # torch float64: the reference stores var = biased variance + eps, torch adds eps itself
+    xt = torch.from_numpy(x).double()
+    ref = torch.nn.functional.batch_norm(xt, None, None, torch.from_numpy(gamma).double(), torch.from_numpy(beta).double(),
+                                         training=True, eps=float(eps)).numpy().ravel()
+    m64, v64 = oracle.batch_mean_var(S, C, N, eps, xf)
+    got64 = oracle.batch_norm_affine(S, C, N, xf, m64.astype(F32), v64.astype(F32), gamma, beta, f64=True)
+    np.testing.assert_allclose(got64, ref, rtol=2e-6, atol=2e-6)   # mean / var were rounded to f32 on the way in
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+    # gamma 1, beta 0 is batch_norm itself, bit for bit (fma(y, 1, 0) == y)
+    same = oracle.batch_norm_affine(S, C, N, xf, mean, var, np.ones(C, F32), np.zeros(C, F32))
+    assert np.array_equal(same.view(np.uint32), (yn + F32(0)).view(np.uint32))
+    # swapped gamma / beta would give this instead
+    swapped = oracle.batch_norm_affine(S, C, N, xf, mean, var, beta, gamma)
+    assert not np.allclose(swapped, got)
+
+
+def test_sum_packed_ten_ones_and_float64_sum(oracle):
+    # tests/test_gpu.rs:302-353: ten arrays of ones joined by a sum give 10.0 in every element; the packed sum of
+    # ten ones is the same 10.0
+    assert oracle.sum_packed(np.ones(10, F32)) == 10.0
+    assert oracle.sum_packed(np.zeros(0, F32)) == 0.0
+    x = (rng(43).standard_normal(100003) * 1e3).astype(F32)
+    assert oracle.sum_packed(x) == pytest.approx(math.fsum(float(v) for v in x), rel=1e-15)
+    # a sum carried in float32 is off by far more than that
+    assert abs(float(np.cumsum(x, dtype=F32)[-1]) - math.fsum(float(v) for v in x)) > 1e-3
+    # integers below 2^24: exact
+    assert oracle.sum_packed(np.arange(5000, dtype=F32)) == 5000 * 4999 / 2
+
+
+def test_online_add_is_a_single_rounded_fma(oracle):
+    # src/ops_gpu.rs:5886: y <- y + rate * x.  Exact rationals: one rounding, operands in this order
+    g = rng(44)
+    x = g.standard_normal(300).astype(F32)
+    y = g.standard_normal(300).astype(F32)
+    for rate in (0.1, -0.75, 1e-3, 3.0):
+        got = oracle.online_add(rate, x, y)
+        r = Fraction(float(F32(rate)))
+        want = np.array([_round_fraction_to_f32(r * Fraction(float(a)) + Fraction(float(b))) for a, b in zip(x, y)], F32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        unfused = (F32(rate) * x + y).astype(F32)
+        assert np.max(np.abs(unfused.astype(np.float64) - got)) <= 1e-6
+    assert np.any((F32(0.1) * x + y).astype(F32) != oracle.online_add(0.1, x, y))   # the fusion is observable
+    # it is not the running-average form (rate 1 would return x) nor the discount form (rate 0 would return x)
+    assert np.array_equal(oracle.online_add(1.0, x, y), (x + y).astype(F32))
+    assert np.array_equal(oracle.online_add(0.0, x, y), y)
+    # three steps of +0.25 from zero: 0.25, 0.5, 0.75 exactly
+    acc = np.zeros(17, F32)
+    for k in range(1, 4):
+        acc = oracle.online_add(0.25, np.ones(17, F32), acc)
+        assert np.all(acc == F32(0.25 * k))
+
+
+def test_flat_bcast_rdiv_brute_force_ieee_division(oracle):
+    # src/ops_gpu.rs:9592 (I1ab, I2b -> Oab): y[a,b] = x[a,b] / r[b], a fastest
+    inner, outer = 7, 5
+    g = rng(45)
+    x = g.standard_normal(inner * outer).astype(F32)
+    r = g.uniform(0.5, 3.0, outer).astype(F32)
+    got = oracle.flat_bcast_rdiv(inner, outer, x, r)
+    want = np.empty(inner * outer, F32)
+    for b in range(outer):
+        for a in range(inner):
+            want[a + inner * b] = _round_fraction_to_f32(Fraction(float(x[a + inner * b])) / Fraction(float(r[b])))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # multiplying by a rounded reciprocal is not the same thing
+    recip = (x.reshape(outer, inner) * (F32(1) / r)[:, None]).astype(F32).ravel()
+    xs = g.standard_normal(4096 * 3).astype(F32)
+    rs = g.uniform(0.5, 3.0, 3).astype(F32)
+    assert np.any(oracle.flat_bcast_rdiv(4096, 3, xs, rs) != (xs.reshape(3, 4096) * (F32(1) / rs)[:, None]).astype(F32).ravel())
+    assert np.max(np.abs(recip.astype(np.float64) - got)) < 1e-6
+    # a divisor indexed by the inner index would divide by the wrong element
+    wrong = (x.reshape(outer, inner) / np.resize(r, inner)[None, :]).astype(F32).ravel()
+    assert not np.array_equal(wrong, got)
+    # special values: x/inf = 0, x/0 = inf with the sign of x, 0/0 = NaN
+    sv = oracle.flat_bcast_rdiv(2, 3, np.array([1, -1, 2, -2, 0, 3], F32), np.array([np.inf, 0.0, 0.0], F32))
+    assert sv[0] == 0 and sv[1] == 0 and np.signbit(sv[1]) and sv[2] == np.inf and sv[3] == -np.inf
+    assert np.isnan(sv[4]) and sv[5] == np.inf

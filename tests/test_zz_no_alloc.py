@@ -43,6 +43,48 @@ def _one(oracle, S, C, N, seed, offset=0):
     assert_close(host(var_a), v64, "var vs fp64 oracle")
 
 
+def test_captured_into_a_graph_on_a_stream_without_scratch():
+    # The callers this entry point is for: a stream under HIP graph capture that holds no reduction scratch.  There
+    # the allocating entry point is refused (error 900, nothing enqueued) while this one is captured -- in a fresh
+    # process this is also its first call on the device, so the address of the static array is looked up during the
+    # capture -- and every replay equals the eager result to the bit.  [12544, 8, 16] cuts its channels into several
+    # tiles, so the partial sums do go through the array.
+    lib = load()
+    d = (12544, 8, 16)
+    S, C, N = d
+    assert lib.symbol("anode_gpu_reduce_scratch_bytes")(*d) > 0
+    g = np.random.default_rng(11)
+    x = dev((2 + 3 * g.standard_normal(S * C * N)).astype(F32))
+    mean, var, refused = empty(C), empty(C), empty(C)
+    stream = torch.cuda.Stream()
+    handle = ctypes.c_void_p(stream.cuda_stream)
+    stream.synchronize()
+    lib.symbol("anode_gpu_release_scratch")(handle)      # torch hands out pooled streams: drop what an earlier test left
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        gpu.call("anode_gpu_batch_mean_3d1_packed_f32", *d, x, refused)
+        err_plain = gpu.take_last_error()
+        rc = lib.symbol(NOALLOC)(S, C, N, 1e-5, x.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                 ctypes.byref(gpu.DEFAULT_CONFIG), handle)
+        err = gpu.take_last_error()
+    assert err_plain == 900, err_plain
+    assert rc == 0 and err == 0, (rc, err)
+    want_mean, want_var = empty(C), empty(C)
+    call(PLAIN, S, C, N, 1e-5, x, want_mean, want_var)   # eager, default stream
+    for k in range(3):
+        mean.fill_(float("nan"))
+        var.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bit_exact(host(mean), host(want_mean), f"mean, replay {k}")
+        assert_bit_exact(host(var), host(want_var), f"var, replay {k}")
+        x.mul_(1.5)                                      # eager work between the replays, on changing input
+        call(PLAIN, S, C, N, 1e-5, x, want_mean, want_var)
+    assert np.all(np.isnan(host(refused)))
+    assert lib.symbol("anode_gpu_release_scratch")(handle) == 0   # the stream never got a buffer
+
+
 def test_two_calls_in_a_row_second_smaller(oracle):
     # first call: many tiles per channel (chunk tiles); second: fewer and smaller partial lists in the same array,
     # which still holds the first call's sums
