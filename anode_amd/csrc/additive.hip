@@ -28,49 +28,23 @@ __device__ inline uint32_t quantize_one(float x, float lo, float scale) {
   return uint32_t(q);
 }
 
-// A thread takes four 16-byte groups one workgroup-width apart (every load instruction of the wave is contiguous)
-// and keeps all four loads in flight; the input is read once, hence non-temporal.  Measured 38 us against 57 us for
-// one group per thread at [256,3,224,224]: the narrow side of this kernel is the 4-byte store.
-__global__ __launch_bounds__(kBlock) void quantize_u8x4_kernel(uint32_t n_groups, uint32_t tail, float lo,
-                                                               float scale, const float *__restrict__ x,
-                                                               uint8_t *__restrict__ y) {
-  constexpr int U = 4;
-  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
-  uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
-  const uint64_t base = uint64_t(blockIdx.x) * (kBlock * U) + threadIdx.x;
-  f32x4 v[U];
-#pragma unroll
-  for (int i = 0; i < U; ++i) {
-    const uint64_t g = base + uint64_t(i) * kBlock;
-    if (g < n_groups) v[i] = load_stream<kNtLoad>(&x4[g]);
-  }
-#pragma unroll
-  for (int i = 0; i < U; ++i) {
-    const uint64_t g = base + uint64_t(i) * kBlock;
-    if (g < n_groups) {
-      y4[g] = quantize_one(v[i].x, lo, scale) | (quantize_one(v[i].y, lo, scale) << 8) |
-              (quantize_one(v[i].z, lo, scale) << 16) | (quantize_one(v[i].w, lo, scale) << 24);
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * 4u + threadIdx.x;
-    y[i] = uint8_t(quantize_one(x[i], lo, scale));
-  }
-}
-
-// 16-byte form on both sides: lane l of a wave loads the 16-byte groups j*64 + l (j = 0..3) of the wave's 256, packs
-// each to a dword, and the wave gathers the dwords through LDS so that each lane stores 16 consecutive bytes: four
-// 1 KiB loads and one 1 KiB store per wave, all contiguous.  One tile per workgroup, 4096 elements.
-__global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t n_groups, uint32_t tail, float lo,
-                                                                float scale, const float *__restrict__ x,
-                                                                uint8_t *__restrict__ y) {
+// 16 bytes per lane on both sides: lane l of a wave loads the 16-byte groups j*64 + l (j = 0..3) of the wave's 256,
+// packs each to a dword, and the wave gathers the dwords through LDS so that each lane stores 16 consecutive bytes:
+// four 1 KiB loads and one 1 KiB store per wave, all contiguous, all four loads of a thread in flight together (the
+// input is read once, hence non-temporal).  One tile per workgroup, 4096 elements.  Measured 34.5 us at
+// [256,3,224,224] (57 us with one 16-byte load and one 4-byte store per thread).  `head` elements (0 to 15) come
+// first, one per thread of workgroup 0, so that the 16-byte stores lie on 16-byte boundaries wherever y lies; x is
+// read where it lies.
+__global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t head, uint32_t n_groups, uint32_t tail,
+                                                                float lo, float scale, const float *__restrict__ x_,
+                                                                uint8_t *__restrict__ y_) {
   __shared__ __align__(16) uint32_t lds[kBlock * 4];
-  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
-  uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
+  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x_ + head);
+  uint32_t *y4 = reinterpret_cast<uint32_t *>(y_ + head);
   const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // first group = first output dword
   f32x4 v[4] = {};
-  if (n_groups != 0u) {  // (fewer than four elements: only the tail below has work)
+  if (n_groups != 0u) {  // (fewer than four elements: only the single elements below have work)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       // unconditional (a group past the end reads the last group again; its code is never stored): with a branch
@@ -92,17 +66,10 @@ __global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t n_group
   } else {
     for (uint32_t k = 0; k < 4u && first + k < n_groups; ++k) y4[first + k] = out[k];
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * 4u + threadIdx.x;
-    y[i] = uint8_t(quantize_one(x[i], lo, scale));
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const uint32_t i = threadIdx.x < head ? threadIdx.x : n_groups * 4u + threadIdx.x;
+    y_[i] = uint8_t(quantize_one(x_[i], lo, scale));
   }
-}
-
-__global__ __launch_bounds__(kBlock) void quantize_u8_scalar_kernel(uint32_t len, float lo, float scale,
-                                                                    const float *__restrict__ x,
-                                                                    uint8_t *__restrict__ y) {
-  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) y[i] = uint8_t(quantize_one(x[i], lo, scale));
 }
 
 // ---------------------------------------------------------------------------
@@ -140,69 +107,32 @@ struct FlatMultMap {
   __device__ float accum(const Param &, float l, float r, uint32_t, float old) const { return fmaf(l, r, old); }
 };
 
-// u8 codes -> per-channel affine f32: y = fma(scale[b], float(q), shift[b]).
-// Each lane loads one dword (4 codes) and stores 16 bytes; the channel of the
-// group's first code is found by exact division, then advanced incrementally.
+// u8 codes -> per-channel affine f32: y = fma(scale[b], float(q), shift[b]).  One 16-byte load of 16 codes per
+// lane, the wave's dwords re-dealt through LDS (see wave_deal_dwords), each lane converts the four dwords it is
+// dealt; the channel of a group's first code is found by exact division, then advanced incrementally.  One tile per
+// workgroup, 4096 codes.  `head` elements (0 to 3) come first, one per thread of workgroup 0, so that the groups
+// of y start on a 16-byte boundary wherever y lies; the codes are read where they lie.
 template <int NT>
-__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x4_kernel(uint32_t n_groups, uint32_t tail,
-                                                                       FastDiv div_s, FastDiv div_c,
-                                                                       const float *__restrict__ scale,
-                                                                       const float *__restrict__ shift,
-                                                                       const uint8_t *__restrict__ x,
-                                                                       float *__restrict__ y) {
-  const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
-  f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
-  const uint32_t S = div_s.d, C = div_c.d;
-  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
-    const uint32_t w = x4[g];
-    uint32_t q, s;
-    div_s.divmod(uint32_t(g) * 4u, q, s);  // 4 g < len, which fits 32 bits
-    uint32_t c = q - div_c.div(q) * C;
-    float a = scale[c], b = shift[c];
-    f32x4 r;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      r[k] = fmaf(a, float((w >> (8 * k)) & 0xffu), b);
-      if (k < 3 && ++s == S) {
-        s = 0;
-        c = (c + 1 == C) ? 0 : c + 1;
-        a = scale[c];
-        b = shift[c];
-      }
-    }
-    store_stream<NT>(&y4[g], r);
-  }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * 4u + threadIdx.x;
-    const uint32_t q = div_s.div(i);
-    const uint32_t c = q - div_c.div(q) * C;
-    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
-  }
-}
-
-// The 16-byte form of the same: one 16-byte load of 16 codes per lane, the wave's dwords re-dealt through LDS (see
-// wave_deal_dwords), each lane converts the four dwords it is dealt.  One tile per workgroup, 4096 codes.
-template <int NT>
-__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t n_dwords, uint32_t tail,
+__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t head, uint32_t n_dwords, uint32_t tail,
                                                                         FastDiv div_s, FastDiv div_c,
                                                                         const float *__restrict__ scale,
                                                                         const float *__restrict__ shift,
-                                                                        const uint8_t *__restrict__ x,
-                                                                        float *__restrict__ y) {
+                                                                        const uint8_t *__restrict__ x_,
+                                                                        float *__restrict__ y_) {
   __shared__ __align__(16) uint32_t lds[kBlock * 4];
+  const uint8_t *x = x_ + head;
   const u32x4 *x16 = reinterpret_cast<const u32x4 *>(x);
-  f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
+  f32x4 *y4 = reinterpret_cast<f32x4 *>(y_ + head);
   const uint32_t S = div_s.d, C = div_c.d;
   const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const uint64_t g16 = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
   const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;
   u32x4 v = {0u, 0u, 0u, 0u};
   if (g16 * 4u + 3u < n_dwords) {
-    v = load_stream<kNtLoad>(&x16[g16]);
+    v = load_stream<kNtLoad, 1>(&x16[g16]);
   } else if (g16 * 4u < n_dwords) {
     const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
-    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = x4[g16 * 4u + k];
+    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = load_stream<0, 1>(&x4[g16 * 4u + k]);
   }
   uint32_t w[4];
   wave_deal_dwords(v, lds + wave * (kWave * 4), w);
@@ -215,7 +145,7 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t
     const uint64_t d = wave_first + uint32_t(j) * kWave + lane;
     const uint32_t dc = (d < n_dwords) ? uint32_t(d) : (n_dwords != 0u ? n_dwords - 1u : 0u);
     uint32_t q;
-    div_s.divmod(dc * 4u, q, sp4[j]);
+    div_s.divmod(head + dc * 4u, q, sp4[j]);
     c4[j] = q - div_c.div(q) * C;
     a4[j] = scale[c4[j]];
     b4[j] = shift[c4[j]];
@@ -240,25 +170,11 @@ __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t
       store_stream<NT>(&y4[d], r);
     }
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_dwords * 4u + threadIdx.x;
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const uint32_t i = threadIdx.x < head ? threadIdx.x : n_dwords * 4u + threadIdx.x;
     const uint32_t q = div_s.div(i);
     const uint32_t c = q - div_c.div(q) * C;
-    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
-  }
-}
-
-__global__ __launch_bounds__(kBlock) void bcast_dequantize_u8_scalar_kernel(uint32_t len, FastDiv div_s,
-                                                                            FastDiv div_c,
-                                                                            const float *__restrict__ scale,
-                                                                            const float *__restrict__ shift,
-                                                                            const uint8_t *__restrict__ x,
-                                                                            float *__restrict__ y) {
-  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) {
-    const uint32_t q = div_s.div(uint32_t(i));  // i < len, which fits 32 bits
-    const uint32_t c = q - div_c.div(q) * div_c.d;
-    y[i] = fmaf(scale[c], float(x[i]), shift[c]);
+    y_[i] = fmaf(scale[c], float(x_[i]), shift[c]);
   }
 }
 
@@ -475,17 +391,11 @@ void launch_quantize(const char *symbol, uint32_t len, float lo, float hi, const
   if (len == 0) return;
   const float scale = (hi - lo) / 255.0f;
   hipStream_t s = as_stream(stream);
-  if (aligned16(x) && aligned16(y)) {
-    const uint32_t groups = len / 4, tail = len % 4;
-    const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
-    quantize_u8x16_kernel<<<blocks ? blocks : 1, kBlock, 0, s>>>(groups, tail, lo, scale, x, y);
-  } else if (aligned16(x) && aligned4(y)) {
-    const uint32_t groups = len / 4, tail = len % 4;
-    const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
-    quantize_u8x4_kernel<<<blocks ? blocks : 1, kBlock, 0, s>>>(groups, tail, lo, scale, x, y);
-  } else {
-    quantize_u8_scalar_kernel<<<stream_grid(len, 1), kBlock, 0, s>>>(len, lo, scale, x, y);
-  }
+  uint32_t head = uint32_t((16u - (reinterpret_cast<uintptr_t>(y) & 15u)) & 15u);  // bytes = elements of y
+  if (head > len) head = len;
+  const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
+  const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
+  quantize_u8x16_kernel<<<blocks ? blocks : 1, kBlock, 0, s>>>(head, groups, tail, lo, scale, x, y);
   note_launch(symbol);
 }
 
@@ -547,22 +457,13 @@ ANODE_EXPORT void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32
   if (len == 0) return;
   hipStream_t s = as_stream(stream);
   const FastDiv div_s(inner_dim), div_c(bcast_dim);
-  if (aligned16(x) && aligned16(y)) {
-    const uint32_t dwords = len / 4, tail = len % 4;
-    const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
-    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
-      bcast_dequantize_u8x16_kernel<decltype(policy)::value>
-          <<<blocks ? blocks : 1, kBlock, 0, s>>>(dwords, tail, div_s, div_c, scale, shift, x, y);
-    });
-  } else if (aligned4(x) && aligned16(y)) {
-    const uint32_t groups = len / 4, tail = len % 4;
-    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
-      bcast_dequantize_u8x4_kernel<decltype(policy)::value>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, scale, shift, x, y);
-    });
-  } else {
-    bcast_dequantize_u8_scalar_kernel<<<stream_grid(len, 1), kBlock, 0, s>>>(len, div_s, div_c, scale, shift, x, y);
-  }
+  const uint32_t head = head_to_align16(y, len);
+  const uint32_t dwords = (len - head) / 4, tail = (len - head) % 4;
+  const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
+  with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {
+    bcast_dequantize_u8x16_kernel<decltype(policy)::value>
+        <<<blocks ? blocks : 1, kBlock, 0, s>>>(head, dwords, tail, div_s, div_c, scale, shift, x, y);
+  });
   note_launch(__func__);
 }
 
@@ -648,7 +549,7 @@ ANODE_EXPORT int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, 
   // Sizes are checked before anything touches the device, so that a refusal has no side effect; the element count
   // first, as in every other entry point (the tiling below is not planned for counts that do not fit 32 bits).
   (void)checked_len(dim0, dim1, dim2, __func__);
-  const bool ptrs_aligned = aligned16(x);
+  const bool ptrs_aligned = true;  // (16-byte loads from any 4-byte aligned address, as in launch_chan_reduce)
   const ReducePlan pl = plan_chan_reduce(dim0, dim1, dim2, ptrs_aligned, uint32_t(tuning().reduce_wg_target),
                                          MeanVarReduce::NIN);
   const size_t need = chan_reduce_scratch_bytes(pl, MeanVarReduce::NACC);
@@ -752,7 +653,7 @@ ANODE_EXPORT void anode_gpu_arg_max_packed_u32(uint32_t dim0, uint32_t dim1, con
   uint32_t blocks = (dim1 + waves_per_block - 1) / waves_per_block;
   const uint32_t cap = 1u << 24;  // one row per wave; the kernel loops only beyond that
   if (blocks > cap) blocks = cap;
-  if (dim0 % 4u == 0 && aligned16(x)) {
+  if (dim0 % 4u == 0) {  // (16-byte loads from any 4-byte aligned address)
     const int nt = stream_policy(size_t(dim0) * dim1 * sizeof(float), tuning().reduce_nontemporal) & kNtLoad;
     if (nt) {
       arg_max_rows_kernel<true, kNtLoad><<<blocks, kBlock, 0, as_stream(stream)>>>(dim0, dim1, x, index);

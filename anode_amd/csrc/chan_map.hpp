@@ -7,7 +7,9 @@
 // element), and the (s, c) pair is then advanced incrementally inside the
 // group, reloading the per-channel parameters only when a channel boundary is
 // crossed.  This keeps full 16-byte accesses for every S, including S that is
-// not a multiple of 4 (7x7 feature maps) and S == 1.
+// not a multiple of 4 (7x7 feature maps) and S == 1, and for arrays that start
+// at any element (a head of up to three elements is peeled so that the stores
+// lie on 16-byte boundaries; the inputs are read where they lie).
 #pragma once
 
 #include "common.hpp"
@@ -51,89 +53,75 @@ __device__ inline float chan_map_apply(const Op &op, const P &p, float x, float 
 // PAIR selects how a group that crosses a channel boundary gets its second parameter set: fetched up front beside
 // the first (channels of a few dozen elements, where a quarter of the groups cross), or on demand while walking
 // the group (long channels, where almost none does and the extra fetch and selects only cost issue slots).
-template <typename V, int NIN, bool ACC, int UNROLL, int NT, bool PAIR, typename Op>
-__global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t n_groups, uint32_t tail, FastDiv div_s,
-                                                          FastDiv div_c, Op op, const float *a_,
+// `head` single elements (0 to 3) come before the groups, `tail` after them, both handled by workgroup 0: the
+// host picks head so that the groups of `out_` start on a 16-byte boundary wherever the array lies; the inputs are
+// read where they lie (4-byte aligned 16-byte loads).
+template <int NIN, bool ACC, int NT, bool PAIR, typename Op>
+__global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t head, uint32_t n_groups, uint32_t tail,
+                                                          FastDiv div_s, FastDiv div_c, Op op, const float *a_,
                                                           const float *b_, const float *c_, float *out_) {
-  constexpr int L = VecLanes<V>::n;
-  const V *a = reinterpret_cast<const V *>(a_);
-  const V *b = reinterpret_cast<const V *>(b_);
-  const V *c3 = reinterpret_cast<const V *>(c_);
-  V *out = reinterpret_cast<V *>(out_);
+  typedef f32x4 V;
+  constexpr int L = 4;
+  const V *a = reinterpret_cast<const V *>(a_ + head);
+  const V *b = reinterpret_cast<const V *>(b_ + head);
+  const V *c3 = reinterpret_cast<const V *>(c_ + head);
+  V *out = reinterpret_cast<V *>(out_ + head);
   const uint32_t S = div_s.d, C = div_c.d;
-  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
-    V va[UNROLL], vb[UNROLL], vc[UNROLL], vo[UNROLL];
+  // one group per thread on a full grid; the loop only runs more than once under the grid cap of the tuning hook
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
+    V va, vb, vc, vo;
+    if (NIN >= 1) va = load_stream<NT>(&a[g]);
+    if (NIN >= 2) vb = load_stream<NT>(&b[g]);
+    if (NIN >= 3) vc = load_stream<NT>(&c3[g]);
+    if (ACC) vo = load_stream<NT>(&out[g]);
+    uint32_t q, s;
+    div_s.divmod(head + uint32_t(g) * uint32_t(L), q, s);
+    uint32_t c = q - div_c.div(q) * C;
+    V r;
+    if (PAIR) {  // the host guarantees S >= L here
+      // A group spans at most two channels.  Both parameter sets are fetched up front, next to the element
+      // loads, so that a group that crosses a channel boundary does not wait for a second, dependent fetch
+      // (with S = 49 a quarter of the groups cross).
+      const uint32_t room = S - s;  // elements of the group that still belong to channel c
+      const typename Op::Param p0 = op.load(c);
+      const uint32_t c1 = (c + 1 == C) ? 0 : c + 1;
+      // (fetched without a branch, from channel c again where the group does not cross: a branch round the
+      // fetch would make it wait for the loads issued before it)
+      const typename Op::Param p1 = op.load(room < uint32_t(L) ? c1 : c);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      // unconditional (a slot past the end reads the last group again and is not stored): with a branch round
-      // each load the compiler waits for the previous load before it issues the next one
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      const uint64_t gc = g < n_groups ? g : uint64_t(n_groups) - 1u;
-      if (NIN >= 1) va[u] = load_stream<NT>(&a[gc]);
-      if (NIN >= 2) vb[u] = load_stream<NT>(&b[gc]);
-      if (NIN >= 3) vc[u] = load_stream<NT>(&c3[gc]);
-      if (ACC) vo[u] = load_stream<NT>(&out[gc]);
-    }
+      for (int k = 0; k < L; ++k) {
+        const bool first = uint32_t(k) < room;
+        const float x = (NIN >= 1) ? va[k] : 0.0f;
+        const float y = (NIN >= 2) ? vb[k] : 0.0f;
+        const float z = (NIN >= 3) ? vc[k] : 0.0f;
+        const float old = ACC ? vo[k] : 0.0f;
+        const typename Op::Param pk = first ? p0 : p1;
+        const uint32_t sk = first ? s + uint32_t(k) : uint32_t(k) - room;
+        r[k] = chan_map_apply<NIN, ACC>(op, pk, x, y, z, sk, old);
+      }
+    } else {
+      // channels shorter than a group: walk (s, c) element by element
+      typename Op::Param p = op.load(c);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) {
-        uint32_t q, s;
-        div_s.divmod(uint32_t(g) * uint32_t(L), q, s);
-        uint32_t c = q - div_c.div(q) * C;
-        V r;
-        if (PAIR) {  // the host guarantees S >= L here
-          // A group spans at most two channels.  Both parameter sets are fetched up front, next to the element
-          // loads, so that a group that crosses a channel boundary does not wait for a second, dependent fetch
-          // (with S = 49 a quarter of the groups cross).
-          const uint32_t room = S - s;  // elements of the group that still belong to channel c
-          const typename Op::Param p0 = op.load(c);
-          const uint32_t c1 = (c + 1 == C) ? 0 : c + 1;
-          // (fetched without a branch, from channel c again where the group does not cross: a branch round the
-          // fetch would make it wait for the loads issued before it)
-          const typename Op::Param p1 = op.load(room < uint32_t(L) ? c1 : c);
-#pragma unroll
-          for (int k = 0; k < L; ++k) {
-            const bool first = uint32_t(k) < room;
-            const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
-            const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
-            const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
-            const float old = ACC ? lane_get<V>(vo[u], k) : 0.0f;
-            if (L == 1) {
-              lane_set<V>(r, k, chan_map_apply<NIN, ACC>(op, p0, x, y, z, s, old));
-            } else {
-              const typename Op::Param pk = first ? p0 : p1;
-              const uint32_t sk = first ? s + uint32_t(k) : uint32_t(k) - room;
-              lane_set<V>(r, k, chan_map_apply<NIN, ACC>(op, pk, x, y, z, sk, old));
-            }
-          }
-        } else {
-          // channels shorter than a group: walk (s, c) element by element
-          typename Op::Param p = op.load(c);
-#pragma unroll
-          for (int k = 0; k < L; ++k) {
-            const float x = (NIN >= 1) ? lane_get<V>(va[u], k) : 0.0f;
-            const float y = (NIN >= 2) ? lane_get<V>(vb[u], k) : 0.0f;
-            const float z = (NIN >= 3) ? lane_get<V>(vc[u], k) : 0.0f;
-            const float v = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? lane_get<V>(vo[u], k) : 0.0f);
-            lane_set<V>(r, k, v);
-            if (k + 1 < L) {
-              if (++s == S) {
-                s = 0;
-                c = (c + 1 == C) ? 0 : c + 1;
-                p = op.load(c);
-              }
-            }
+      for (int k = 0; k < L; ++k) {
+        const float x = (NIN >= 1) ? va[k] : 0.0f;
+        const float y = (NIN >= 2) ? vb[k] : 0.0f;
+        const float z = (NIN >= 3) ? vc[k] : 0.0f;
+        r[k] = chan_map_apply<NIN, ACC>(op, p, x, y, z, s, ACC ? vo[k] : 0.0f);
+        if (k + 1 < L) {
+          if (++s == S) {
+            s = 0;
+            c = (c + 1 == C) ? 0 : c + 1;
+            p = op.load(c);
           }
         }
-        store_stream<NT>(&out[g], r);
       }
     }
+    store_stream<NT>(&out[g], r);
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * uint32_t(L) + threadIdx.x;
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const uint32_t i = threadIdx.x < head ? threadIdx.x : n_groups * uint32_t(L) + threadIdx.x;
     uint32_t q, s;
     div_s.divmod(i, q, s);
     const uint32_t c = q - div_c.div(q) * C;
@@ -228,22 +216,20 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
       chan_map_cols_kernel<NIN, ACC, NT, Op><<<uint32_t((threads + kBlock - 1) / kBlock), kBlock, 0, s>>>(
           S, N, uint32_t(threads), div_gpp, div_s, op, a, b, c, out);
     });
-  } else if (vec) {
-    const uint32_t groups = len / 4, tail = len % 4;
+  } else {
+    const uint32_t head = head_to_align16(out, len);
+    const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
     const bool pair = S >= 4 && S < 4096;
     with_stream_policy(nt, [&](auto policy) {
       constexpr int NT = decltype(policy)::value;
       if (pair) {
-        chan_map_kernel<f32x4, NIN, ACC, 1, NT, true, Op>
-            <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+        chan_map_kernel<NIN, ACC, NT, true, Op>
+            <<<stream_grid(groups ? groups : 1, 1), kBlock, 0, s>>>(head, groups, tail, div_s, div_c, op, a, b, c, out);
       } else {
-        chan_map_kernel<f32x4, NIN, ACC, 1, NT, false, Op>
-            <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, div_s, div_c, op, a, b, c, out);
+        chan_map_kernel<NIN, ACC, NT, false, Op>
+            <<<stream_grid(groups ? groups : 1, 1), kBlock, 0, s>>>(head, groups, tail, div_s, div_c, op, a, b, c, out);
       }
     });
-  } else {
-    chan_map_kernel<float, NIN, ACC, 4, 0, false, Op>
-        <<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, div_s, div_c, op, a, b, c, out);
   }
   note_launch(symbol);
 }

@@ -2,12 +2,12 @@
 // join, u8 -> 32-bit widening (upcast, dequantize) and the additive f32 -> u8
 // quantiser.
 //
-// Data path: every lane moves 16 bytes per access (global_load/store_dwordx4),
-// consecutive lanes touch consecutive 16-byte groups, and each thread keeps
-// UNROLL independent groups in flight before the first store.  Arrays whose
-// pointers are not 16-byte aligned take the same kernels with one element per
-// lane.  All maps read an element before writing the same index, so an output
-// that aliases an input at equal index is safe.
+// Data path: every lane moves 16 bytes per access (global_load/store_dwordx4) and
+// consecutive lanes touch consecutive 16-byte groups.  Arrays may start at any
+// element: up to three head elements are peeled so that the stores lie on
+// 16-byte boundaries, and the loads are issued where the inputs lie.  All maps
+// read an element before writing the same index, so an output that aliases an
+// input at equal index is safe.
 #include "common.hpp"
 
 #include <cmath>
@@ -68,12 +68,6 @@ struct LogisticBwdMap { __device__ float operator()(float dy, float y) const { r
 // flat_join.cu:31-35: a = x1, b = x2
 struct CopyUnitStepProductJoin { __device__ float operator()(float x1, float x2) const { return x1 * float(x2 > 0.0f); } };
 
-template <typename V> struct Lanes;
-template <> struct Lanes<float> { static constexpr int n = 1; };
-template <> struct Lanes<f32x4> { static constexpr int n = 4; };
-
-template <typename Op>
-__device__ inline float apply_vec(const Op &op, float a, float b) { return op(a, b); }
 template <typename Op>
 __device__ inline f32x4 apply_vec(const Op &op, f32x4 a, f32x4 b) {
   f32x4 r;
@@ -84,37 +78,28 @@ __device__ inline f32x4 apply_vec(const Op &op, f32x4 a, f32x4 b) {
   return r;
 }
 
-// n_groups groups of Lanes<V>::n elements, then `tail` single elements that
-// start at element n_groups * Lanes<V>::n (handled by workgroup 0).
-template <typename V, int NIN, int UNROLL, int NT, typename Op>
-__global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t n_groups, uint32_t tail, Op op,
-                                                          const float *a_, const float *b_,
-                                                          float *out_) {
+// `head` single elements, then n_groups groups of four, then `tail` single elements; the single elements are
+// handled by workgroup 0.  The host picks head so that the groups of `out_` start on a 16-byte boundary; the inputs
+// are read where they lie (4-byte aligned 16-byte loads).
+template <int NIN, int NT, typename Op>
+__global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t head, uint32_t n_groups, uint32_t tail, Op op,
+                                                          const float *a_, const float *b_, float *out_) {
   // no __restrict__: out_ may alias a_ or b_ at equal index
-  const V *a = reinterpret_cast<const V *>(a_);
-  const V *b = reinterpret_cast<const V *>(b_);
-  V *out = reinterpret_cast<V *>(out_);
-  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
-    V va[UNROLL], vb[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      // unconditional (a slot past the end reads the last group again and is not stored): with a branch round
-      // each load the compiler waits for the previous load before it issues the next one
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      const uint64_t gc = g < n_groups ? g : uint64_t(n_groups) - 1u;
-      va[u] = load_stream<NT>(&a[gc]);
-      vb[u] = (NIN == 2) ? load_stream<NT>(&b[gc]) : va[u];
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) store_stream<NT>(&out[g], apply_vec(op, va[u], vb[u]));
-    }
+  const f32x4 *a = reinterpret_cast<const f32x4 *>(a_ + head);
+  const f32x4 *b = reinterpret_cast<const f32x4 *>(b_ + head);
+  f32x4 *out = reinterpret_cast<f32x4 *>(out_ + head);
+  // one 16-byte group per thread on a full grid: measured faster on MI355X than any unrolled persistent loop
+  // (two or four groups per thread on a correspondingly smaller grid, all their loads in flight together, run at
+  // 6.1 TB/s against 6.65 for the copy of 822 MB arrays); the loop only runs more than once under the grid cap of
+  // the tuning hook
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  for (uint64_t g = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g < n_groups; g += stride) {
+    const f32x4 va = load_stream<NT>(&a[g]);
+    const f32x4 vb = (NIN == 2) ? load_stream<NT>(&b[g]) : va;
+    store_stream<NT>(&out[g], apply_vec(op, va, vb));
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * uint32_t(Lanes<V>::n) + threadIdx.x;
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const uint32_t i = threadIdx.x < head ? threadIdx.x : n_groups * 4u + threadIdx.x;  // (head + 4 * n_groups + (t - head))
     const float x = a_[i];
     const float y = (NIN == 2) ? b_[i] : x;
     out_[i] = op(x, y);
@@ -126,21 +111,14 @@ void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, co
                      CUstream_st *stream) {
   if (len == 0) return;
   const Tuning &t = tuning();
-  const bool vec = aligned16(a) && aligned16(out) && (NIN == 1 || aligned16(b));
   hipStream_t s = as_stream(stream);
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
-  if (vec) {
-    // one 16-byte group per thread: measured faster on MI355X than any unrolled persistent loop
-    const uint32_t groups = len / 4, tail = len % 4;
-    // (Two or four groups per thread on a correspondingly smaller grid, all their loads in flight together, run at
-    // 6.1 TB/s against 6.65 for the copy of 822 MB arrays.)
-    with_stream_policy(nt, [&](auto policy) {
-      flat_map_kernel<f32x4, NIN, 1, decltype(policy)::value, Op>
-          <<<stream_grid(groups, 1), kBlock, 0, s>>>(groups, tail, op, a, b, out);
-    });
-  } else {
-    flat_map_kernel<float, NIN, 4, 0, Op><<<stream_grid(len, 4), kBlock, 0, s>>>(len, 0, op, a, b, out);
-  }
+  const uint32_t head = head_to_align16(out, len);
+  const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
+  with_stream_policy(nt, [&](auto policy) {
+    flat_map_kernel<NIN, decltype(policy)::value, Op>
+        <<<stream_grid(groups ? groups : 1, 1), kBlock, 0, s>>>(head, groups, tail, op, a, b, out);
+  });
   note_launch(symbol);
 }
 
@@ -159,64 +137,29 @@ struct DequantizeOp {
   __device__ float operator()(uint32_t q) const { return fmaf(float(q), scale, lo); }
 };
 
-// Vector form: each lane loads one dword (4 codes) and stores 16 bytes, so a
-// wave reads 256 contiguous bytes and writes 1 KiB contiguous bytes per access.
-template <int UNROLL, int NT, typename Op>
-__global__ __launch_bounds__(kBlock) void widen_u8x4_kernel(uint32_t n_groups, uint32_t tail, Op op,
-                                                            const uint8_t *__restrict__ x,
-                                                            typename Op::out_t *__restrict__ y) {
-  typedef typename Op::out4_t O4;
-  const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
-  O4 *y4 = reinterpret_cast<O4 *>(y);
-  constexpr uint32_t kTile = uint32_t(UNROLL) * kBlock;
-  const uint64_t stride = uint64_t(gridDim.x) * kTile;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t base = uint64_t(blockIdx.x) * kTile; base < n_groups; base += stride) {
-    uint32_t w[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) w[u] = load_stream<NT>(&x4[g]);
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const uint64_t g = base + uint64_t(u) * kBlock + threadIdx.x;
-      if (g < n_groups) {
-        O4 r;
-        r.x = op(w[u] & 0xffu);
-        r.y = op((w[u] >> 8) & 0xffu);
-        r.z = op((w[u] >> 16) & 0xffu);
-        r.w = op(w[u] >> 24);
-        store_stream<NT>(&y4[g], r);
-      }
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_groups * 4u + threadIdx.x;
-    y[i] = op(uint32_t(x[i]));
-  }
-}
-
-// 16-byte form: each lane loads 16 codes in one access, the wave re-deals the dwords through LDS, and each lane
-// converts the four dwords it is dealt, so that every load (1 KiB) and every store (four of 1 KiB) of the wave is
-// contiguous.  One tile per workgroup, 4096 codes.  Measured 34.7 us against 35.8 us for the dword form at
-// [256,3,224,224].
+// Each lane loads 16 codes in one access, the wave re-deals the dwords through LDS, and each lane converts the
+// four dwords it is dealt, so that every load (1 KiB) and every store (four of 1 KiB) of the wave is contiguous.
+// One tile per workgroup, 4096 codes.  Measured 34.7 us against 35.8 us for a form with one dword per lane at
+// [256,3,224,224].  `head` elements (0 to 3) come first, one per thread of workgroup 0, so that the groups of y
+// start on a 16-byte boundary wherever y lies; the codes are read where they lie (byte-aligned 16-byte loads).
 template <int NT, typename Op>
-__global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t n_dwords, uint32_t tail, Op op,
-                                                             const uint8_t *__restrict__ x,
-                                                             typename Op::out_t *__restrict__ y) {
+__global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t head, uint32_t n_dwords, uint32_t tail, Op op,
+                                                             const uint8_t *__restrict__ x_,
+                                                             typename Op::out_t *__restrict__ y_) {
   typedef typename Op::out4_t O4;
   __shared__ __align__(16) uint32_t lds[kBlock * 4];
+  const uint8_t *x = x_ + head;
   const u32x4 *x16 = reinterpret_cast<const u32x4 *>(x);
-  O4 *y4 = reinterpret_cast<O4 *>(y);
+  O4 *y4 = reinterpret_cast<O4 *>(y_ + head);
   const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const uint64_t g16 = uint64_t(blockIdx.x) * kBlock + threadIdx.x;  // this lane's group of 16 codes
   const uint64_t wave_first = (uint64_t(blockIdx.x) * kBlock + uint64_t(wave) * kWave) * 4u;  // the wave's first dword
   u32x4 v = {0u, 0u, 0u, 0u};
   if (g16 * 4u + 3u < n_dwords) {
-    v = load_stream<kNtLoad>(&x16[g16]);  // the codes are read once, whatever the size
+    v = load_stream<kNtLoad, 1>(&x16[g16]);  // the codes are read once, whatever the size
   } else if (g16 * 4u < n_dwords) {  // the last, partial group of the array: dword by dword
     const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
-    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = x4[g16 * 4u + k];
+    for (uint32_t k = 0; k < 4u && g16 * 4u + k < n_dwords; ++k) v[k] = load_stream<0, 1>(&x4[g16 * 4u + k]);
   }
   uint32_t w[4];
   wave_deal_dwords(v, lds + wave * (kWave * 4), w);
@@ -232,18 +175,10 @@ __global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t n_dwords, 
       store_stream<NT>(&y4[d], r);
     }
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail) {
-    const uint32_t i = n_dwords * 4u + threadIdx.x;
-    y[i] = op(uint32_t(x[i]));
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const uint32_t i = threadIdx.x < head ? threadIdx.x : n_dwords * 4u + threadIdx.x;
+    y_[i] = op(uint32_t(x_[i]));
   }
-}
-
-template <typename Op>
-__global__ __launch_bounds__(kBlock) void widen_u8_scalar_kernel(uint32_t len, Op op,
-                                                                 const uint8_t *__restrict__ x,
-                                                                 typename Op::out_t *__restrict__ y) {
-  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < len; i += stride) y[i] = op(uint32_t(x[i]));
 }
 
 template <typename Op>
@@ -252,26 +187,14 @@ void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, 
   if (len == 0) return;
   const Tuning &t = tuning();
   hipStream_t s = as_stream(stream);
-  if (aligned16(x) && aligned16(y)) {
-    const uint32_t dwords = len / 4, tail = len % 4;
-    const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
-    // the policy looks at the output, which is four times the input
-    const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
-    with_stream_policy(nt, [&](auto policy) {
-      widen_u8x16_kernel<decltype(policy)::value, Op><<<blocks ? blocks : 1, kBlock, 0, s>>>(dwords, tail, op, x, y);
-    });
-  } else if (aligned4(x) && aligned16(y)) {
-    const uint32_t groups = len / 4, tail = len % 4;
-    // the store policy looks at the output, which is four times the input
-    const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
-    // two groups per thread: with 4-byte loads a thread needs more than one in flight (41 us against 44 us at
-    // [256,3,224,224])
-    with_stream_policy(nt, [&](auto policy) {
-      widen_u8x4_kernel<2, decltype(policy)::value, Op><<<stream_grid(groups, 2), kBlock, 0, s>>>(groups, tail, op, x, y);
-    });
-  } else {
-    widen_u8_scalar_kernel<Op><<<stream_grid(len, 1), kBlock, 0, s>>>(len, op, x, y);
-  }
+  const uint32_t head = head_to_align16(y, len);
+  const uint32_t dwords = (len - head) / 4, tail = (len - head) % 4;
+  const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
+  // the policy looks at the output, which is four times the input
+  const int nt = stream_policy(size_t(len) * 4, t.nontemporal);
+  with_stream_policy(nt, [&](auto policy) {
+    widen_u8x16_kernel<decltype(policy)::value, Op><<<blocks ? blocks : 1, kBlock, 0, s>>>(head, dwords, tail, op, x, y);
+  });
   note_launch(symbol);
 }
 

@@ -133,7 +133,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const uint32_t g = threadIdx.x + uint32_t(i) * kBlock;
-        in[i] = reinterpret_cast<const f32x4 *>(xt)[g < n4 ? g : n4 - 1u];
+        in[i] = load_stream<0>(reinterpret_cast<const f32x4 *>(xt) + (g < n4 ? g : n4 - 1u));
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kRowStreamThreads) __attribute__((amdgpu_waves_per_
       const uint32_t gc = g < rg.groups ? uint32_t(g) : rg.groups - 1u;
       if (VEC) {
         const f32x4 q = decltype(last_use)::value ? load_stream<NT>(reinterpret_cast<const f32x4 *>(rg.xa + size_t(gc) * 4u))
-                                                  : *reinterpret_cast<const f32x4 *>(rg.xa + size_t(gc) * 4u);
+                                                  : load_stream<0>(reinterpret_cast<const f32x4 *>(rg.xa + size_t(gc) * 4u));
 #pragma unroll
         for (int j = 0; j < W; ++j) t[u][j] = q[j];
       } else {
@@ -698,7 +698,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
     const size_t lds_bytes = size_t(rows_per_block) * K * sizeof(float);
     const FastDiv div_kj(KJ);
     const uint32_t rot = pick_row_rotation(K, log2g);
-    const int vec = (aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx))) ? 1 : 0;
+    const int vec = 1;  // 16-byte copies between the arrays and the tile, wherever the arrays lie (4-byte aligned accesses)
     with_stream_policy(nt & kNtStore, [&](auto policy) {
       constexpr int NT = decltype(policy)::value;
       auto launch = [&](auto kmax, auto lg) {
@@ -737,8 +737,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
         with_kmax_wide(std::integral_constant<int, 3>{});
       }
     });
-  } else if (K <= 2048 && K > 512 && R <= 2u * uint32_t(device_cu_count()) && (K % 4u == 0) && aligned16(x) &&
-             aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx))) {
+  } else if (K <= 2048 && K > 512 && R <= 2u * uint32_t(device_cu_count()) && (K % 4u == 0)) {
     // few rows: a workgroup per row instead of a wave, so that every CU has work ([256, 1000], launch-bound:
     // softmax + NLL + backward 8.2 -> 7.4 us as three launches inside a graph, 4.3 -> 3.8 us as one)
     with_stream_policy(nt, [&](auto policy) {
@@ -751,7 +750,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   } else if (K <= 2048) {
     uint32_t blocks = (R + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > max_blocks) blocks = max_blocks;
-    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx));
+    const bool vec = (K % 4u == 0);  // rows of whole 16-byte groups, wherever the arrays lie
 #define ANODE_ROW_WAVE(VPL)                                                              \
   do {                                                                                   \
     if (vec) {                                                                           \
@@ -774,7 +773,7 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
 #undef ANODE_ROW_WAVE
   } else {
     const uint32_t blocks = R < max_blocks ? R : max_blocks;
-    const bool vec = (K % 4u == 0) && aligned16(x) && aligned16(y) && (nl.dx == nullptr || aligned16(nl.dx));
+    const bool vec = (K % 4u == 0);  // rows of whole 16-byte groups, wherever the arrays lie
 #define ANODE_ROW_BLOCKREG(VPT)                                                          \
   do {                                                                                   \
     if (vec) {                                                                           \
@@ -957,9 +956,9 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     // the labels and the upstream gradient are requested first, so that they are there when the classes are
     U lab;
-    if (NLL) lab = *reinterpret_cast<const U *>(cat + pix);
+    if (NLL) lab = load_stream<0>(reinterpret_cast<const U *>(cat + pix));
     V d;
-    if (BWD) d = *reinterpret_cast<const V *>(dy + pix);
+    if (BWD) d = load_stream<0>(reinterpret_cast<const V *>(dy + pix));
     if (NLL) issue_order_fence();
     // Every slot is loaded, a slot past the last class from the last class's plane again (and set to -inf below):
     // with a branch round each load the compiler waits for the previous load before it issues the next one.
@@ -1039,7 +1038,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
           const float pr = lane_get<V>(pick, w) * lane_get<V>(inv, w);
           lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr) : (pg.ignore ? 0.0f : __builtin_nanf("")));
         }
-        *reinterpret_cast<V *>(nll + pix) = out;
+        store_stream<0>(reinterpret_cast<V *>(nll + pix), out);
       }
     }
   }
@@ -1060,7 +1059,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_reg_kernel(PixelGrid pg, co
 // nd_pair_offsets_fit()), uint64_t otherwise (samples of a gigabyte and more), which costs the scalar base.
 template <typename OFF>
 __device__ inline f32x4 load_lane_off(const float *wave_base, OFF off, std::integral_constant<int, 0>) {
-  return *reinterpret_cast<const f32x4 *>(reinterpret_cast<const char *>(wave_base) + off);
+  return load_stream<0>(reinterpret_cast<const f32x4 *>(reinterpret_cast<const char *>(wave_base) + off));
 }
 template <typename OFF>
 __device__ inline f32x4 load_lane_off(const float *wave_base, OFF off, std::integral_constant<int, kNtLoad>) {
@@ -1106,9 +1105,9 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_pair_kernel(PixelGrid pg, c
   const uint32_t last_even = (pg.C - 1u) & ~1u;
   // the labels and the upstream gradient are requested first, so that they are there when the classes are
   u32x4 lab;
-  if (NLL) lab = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(cat + pix_wave) + off_pix);
+  if (NLL) lab = load_stream<0>(reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(cat + pix_wave) + off_pix));
   f32x4 d;
-  if (BWD) d = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const char *>(dy + pix_wave) + off_pix);
+  if (BWD) d = load_stream<0>(reinterpret_cast<const f32x4 *>(reinterpret_cast<const char *>(dy + pix_wave) + off_pix));
   if (NLL) issue_order_fence();
   // Every slot is loaded, a slot past the last class from the last class's plane again (and set to -inf below).
   f32x4 v[H];
@@ -1180,7 +1179,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_pair_kernel(PixelGrid pg, c
         const float pr = pick[w] * inv[w];
         out[w] = lab[w] < pg.C ? -logf(pr) : (pg.ignore ? 0.0f : __builtin_nanf(""));
       }
-      *reinterpret_cast<f32x4 *>(reinterpret_cast<char *>(nll + pix_wave) + off_pix) = out;
+      store_stream<0>(reinterpret_cast<f32x4 *>(reinterpret_cast<char *>(nll + pix_wave) + off_pix), out);
     }
   }
 }
@@ -1220,7 +1219,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
 #pragma unroll
       for (int u = 0; u < U; ++u) {  // a slot past the last class reads the last class again and is set to -inf
         const uint32_t k = k0 + uint32_t(u * SPLIT);
-        v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
+        v[u] = load_stream<0>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u)));
       }
       V bm = PixVec<V>::splat(kNegInf);
 #pragma unroll
@@ -1257,12 +1256,12 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_stream_kernel(PixelGrid pg,
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t k = k0 + uint32_t(u * SPLIT);
-        v[u] = *reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u));
+        v[u] = load_stream<0>(reinterpret_cast<const V *>(x + base + size_t(pg.P) * (k < pg.C ? k : pg.C - 1u)));
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t k = k0 + uint32_t(u * SPLIT);
-        if (k < pg.C) *reinterpret_cast<V *>(y + base + size_t(pg.P) * k) = vexp(v[u] - m) * inv;
+        if (k < pg.C) store_stream<0>(reinterpret_cast<V *>(y + base + size_t(pg.P) * k), V(vexp(v[u] - m) * inv));
       }
     }
   }
@@ -1282,7 +1281,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
     pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
-    const U lab = *reinterpret_cast<const U *>(cat + pix);
+    const U lab = load_stream<0>(reinterpret_cast<const U *>(cat + pix));
     float pr[W];
 #pragma unroll
     for (int w = 0; w < W; ++w) {
@@ -1294,7 +1293,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_kernel(PixelGrid pg
     for (int w = 0; w < W; ++w) {
       lane_set<V>(out, w, lane_get_u(lab, w) < pg.C ? -logf(pr[w]) : (pg.ignore ? 0.0f : __builtin_nanf("")));
     }
-    *reinterpret_cast<V *>(nll + pix) = out;
+    store_stream<0>(reinterpret_cast<V *>(nll + pix), out);
   }
 }
 
@@ -1317,8 +1316,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_kernel(PixelGri
     pixel_decode(pg, uint32_t(g), W, p, n);  // g < total_groups, which fits 32 bits
     const size_t pix = size_t(p) + size_t(pg.P) * n;
     const size_t base = size_t(p) + size_t(pg.P) * pg.C * n;
-    V d = *reinterpret_cast<const V *>(dy + pix);
-    const U lab = *reinterpret_cast<const U *>(cat + pix);
+    V d = load_stream<0>(reinterpret_cast<const V *>(dy + pix));
+    const U lab = load_stream<0>(reinterpret_cast<const U *>(cat + pix));
     if (pg.ignore) {
 #pragma unroll
       for (int w = 0; w < W; ++w) {
@@ -1638,7 +1637,7 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
   const uint32_t max_blocks = 1u << 24;
   if (blocks > max_blocks) blocks = max_blocks;
   const bool starts_aligned = (uint64_t(SB) * slab) % 4u == 0 || N <= SB;
-  const int vec = (starts_aligned && aligned16(x) && aligned16(y) && (!BWD || aligned16(dx))) ? 1 : 0;
+  const int vec = starts_aligned ? 1 : 0;  // (tiles of whole 16-byte groups, wherever the arrays lie)
   const size_t lds_bytes = size_t(SB) * slab * sizeof(float);
   const FastDiv div_p(P), div_c(C);
   // logits in, probabilities (and the gradient) out: all streamed
@@ -1863,8 +1862,10 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
 // exponentials are added, hence the bits of p, depends on the kernel.
 bool nd_one_pixel_per_thread(uint32_t P, uint32_t C, bool vec) { return (!vec || P < 1024) && C > 32 && C <= 128; }
 
-// whether the plain n-d entry point takes its 16-byte kernels: decided by the plane length and by x and y alone
-bool nd_vec_xy(uint32_t P, const float *x, const float *y) { return (P % 4 == 0) && aligned16(x) && aligned16(y); }
+// whether the n-d entry points take their 16-byte kernels: planes of whole 16-byte groups; where the arrays lie
+// does not matter (the accesses only ask for 4-byte alignment), so every entry point picks the same kernel family
+// for a shape and a pixel's sum is added in the same order by all of them
+bool nd_vec(uint32_t P) { return P % 4 == 0; }
 
 void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                        CUstream_st *stream) {
@@ -1875,7 +1876,7 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     return;
   }
   hipStream_t s = as_stream(stream);
-  const bool vec = nd_vec_xy(P, x, y);
+  const bool vec = nd_vec(P);
   const ColTile ct = nd_col_tile(P, C);
   if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
@@ -1917,7 +1918,7 @@ void launch_softmax_nd_cat_nll(const char *symbol, uint32_t P, uint32_t C, uint3
                                const uint32_t *cat, float *nll, CUstream_st *stream, bool ignore) {
   (void)checked_len(P, C, N, symbol);
   if (P == 0 || N == 0) return;
-  if (P % 4 == 0 && aligned16(cat) && aligned16(nll)) {
+  if (P % 4 == 0) {
     PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
     pg.xcd = (tuning().nd_xcd_mask & 4) ? 1u : 0u;
     softmax_nd_cat_nll_kernel<f32x4><<<pixel_blocks(pg.total_groups), kBlock, 0, as_stream(stream)>>>(pg, prob, cat, nll);
@@ -1950,8 +1951,8 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_kernel(uin
     const uint32_t n = div_c.div(plane);
     const uint32_t k = plane - n * C;
     const size_t pix = size_t(n) * P + size_t(r) * 4u;
-    f32x4 d = *reinterpret_cast<const f32x4 *>(dy + pix);
-    const u32x4 lab = *reinterpret_cast<const u32x4 *>(cat + pix);
+    f32x4 d = load_stream<0>(reinterpret_cast<const f32x4 *>(dy + pix));
+    const u32x4 lab = load_stream<0>(reinterpret_cast<const u32x4 *>(cat + pix));
     const f32x4 pr = load_stream<NT>(reinterpret_cast<const f32x4 *>(prob) + g);
     f32x4 old = {0.0f, 0.0f, 0.0f, 0.0f};
     if (ACC) old = load_stream<NT>(reinterpret_cast<const f32x4 *>(dx) + g);
@@ -1991,7 +1992,7 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
     return;
   }
   hipStream_t s = as_stream(stream);
-  const bool vec = (P % 4 == 0) && aligned16(dy) && aligned16(prob) && aligned16(cat) && aligned16(dx);
+  const bool vec = (P % 4 == 0);  // planes of whole 16-byte groups, wherever the arrays lie
   uint32_t chunk = C;
   if (vec && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
     const uint32_t total_groups = len / 4u;
@@ -2114,17 +2115,14 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                         as_stream(stream));
     note_launch(__func__);
-  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0); ct.fits && aligned16(x) && aligned16(softmax)) {
+  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0); ct.fits) {
     launch_softmax_nd_coltile<true, false>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
                                            false, as_stream(stream));
     note_launch(__func__);
-  } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
-                              aligned16(nll);
-             // the kernel family (and with it the order of a pixel's sum) follows x and softmax alone, as in the
-             // plain entry point: where those two allow 16-byte accesses and the label or nll array does not, the
-             // two passes run back to back instead of a kernel that would round differently
-             vec == nd_vec_xy(prefix_dim, x, softmax) &&
-             (dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec)))) {
+  } else if (const bool vec = nd_vec(prefix_dim);
+             // (the kernel family, and with it the order of a pixel's sum, follows the shape alone, here as in the
+             // plain entry point)
+             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
@@ -2156,15 +2154,12 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
                                        as_stream(stream));
     note_launch(__func__);
   } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0);
-             ct.fits && aligned16(x) && aligned16(softmax) && aligned16(dx)) {
+             ct.fits) {
     launch_softmax_nd_coltile<true, true>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                           as_stream(stream));
     note_launch(__func__);
-  } else if (const bool vec = (prefix_dim % 4 == 0) && aligned16(x) && aligned16(softmax) && aligned16(cat_data) &&
-                              aligned16(nll) && aligned16(dy) && aligned16(dx);
-             // (as above: a label, nll, dy or dx array that lies differently sends the call to the three passes)
-             vec == nd_vec_xy(prefix_dim, x, softmax) &&
-             (dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec)))) {
+  } else if (const bool vec = nd_vec(prefix_dim);
+             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
     if (vec) {
       launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);

@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--shape-sweep", action="store_true",
                     help="instead of the benchmark: batch-norm pieces over S x C, row softmax over K and channel-axis "
                          "softmax over C x P, each on ~256 MB arrays, one JSON line (where the tilings switch)")
+    ap.add_argument("--source-fingerprints", action="store_true",
+                    help="print the fingerprints of the kernel sources behind the measured-traffic table and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="add one plain copy of a known size to the step (scale for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
@@ -61,18 +63,62 @@ class Launch:
 # of the profile named in TRAFFIC_SOURCE, not re-measured by this run; a launch that is not listed reports null.
 TRAFFIC_SOURCE = "profiles/bench_step_dominant_kernels_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not re-measured in this run)"
 MEASURED_TRAFFIC = {
-    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2a"): 2466145290,
-    ("anode_gpu_batch_norm_3d1_packed_f32", "bn_fwd_cfg2a"): 1644132867,
-    ("anode_gpu_batch_mean_3d1_packed_f32", "bn_fwd_cfg2b"): 102808380,
-    ("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", "bn_bwd_cfg2b"): 205583995,
-    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): 308430450,
-    ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): 1610539015,
-    ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): 637591035,
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): 291192285,
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): 671287790,
-    ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): 192705077,
-    ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): 192703030,
+    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2a"): (2466145290, "bn_maps"),
+    ("anode_gpu_batch_norm_3d1_packed_f32", "bn_fwd_cfg2a"): (1644132867, "bn_maps"),
+    ("anode_gpu_batch_mean_3d1_packed_f32", "bn_fwd_cfg2b"): (102808380, "bn_reductions"),
+    ("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", "bn_bwd_cfg2b"): (205583995, "bn_reductions"),
+    ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): (308430450, "bn_maps"),
+    ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): (1610539015, "flat_maps"),
+    ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): (637591035, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291192285, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671287790, "softmax"),
+    ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): (192705077, "flat_maps"),
+    ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): (192703030, "flat_maps"),
 }
+# The kernel sources behind each family of the table and their fingerprint when the counters were read (sha256 over
+# the files' bytes, first 16 hex digits).  A figure whose family's sources have changed since is reported as null
+# with a note instead of the stale number: run the two counter passes again, update the table and the fingerprints
+# (`python3 bench.py --source-fingerprints` prints the current ones).
+TRAFFIC_FAMILY_SOURCES = {
+    "bn_maps": ["common.hpp", "chan_map.hpp", "batch_norm.hip"],
+    "bn_reductions": ["common.hpp", "chan_reduce.hpp", "batch_norm.hip"],
+    "flat_maps": ["common.hpp", "flat_map.hip"],
+    "softmax": ["common.hpp", "softmax.hip"],
+}
+TRAFFIC_FAMILY_FINGERPRINT = {
+    "bn_maps": "",
+    "bn_reductions": "",
+    "flat_maps": "",
+    "softmax": "",
+}
+
+
+def source_fingerprints():
+    import hashlib
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "anode_amd", "csrc")
+    out = {}
+    for family, files in TRAFFIC_FAMILY_SOURCES.items():
+        h = hashlib.sha256()
+        try:
+            for f in files:
+                with open(os.path.join(here, f), "rb") as fh:
+                    h.update(fh.read())
+            out[family] = h.hexdigest()[:16]
+        except OSError:
+            out[family] = None
+    return out
+
+
+def measured_traffic(symbol, group, current):
+    """(bytes or None, note or None) for a launch of the table; None/None for a launch that is not in it."""
+    entry = MEASURED_TRAFFIC.get((symbol, group))
+    if entry is None:
+        return None, None
+    nbytes, family = entry
+    if current.get(family) != TRAFFIC_FAMILY_FINGERPRINT.get(family):
+        return None, (f"STALE: the sources of the {family} kernels ({', '.join(TRAFFIC_FAMILY_SOURCES[family])}) have changed "
+                      f"since the counters were read ({nbytes} bytes then); the counter passes must be repeated")
+    return nbytes, None
 
 
 class Draws:
@@ -695,6 +741,47 @@ def cpu_baseline():
         timed("cast", 5 * n_q, lambda: o.dequantize_u8(0.0, 1.0, q))
         timed("cast", 5 * n_q, lambda: o.upcast_u8(q))
 
+    # BASELINE config 0, the configuration named as the CPU reference path: BN fwd+bwd on [32,16,28,28] (the nine
+    # reference launches) and softmax + NLL + backward on [32,10], per pass, on one thread and on all cores
+    def config0(nthreads):
+        o.set_threads(nthreads)
+        S0, C0, N0 = 784, 16, 32
+        d0 = (S0, C0, N0)
+        g0 = np.random.default_rng(0)
+        x0 = g0.standard_normal(S0 * C0 * N0).astype(F32)
+        dy0 = g0.standard_normal(S0 * C0 * N0).astype(F32)
+        lg0 = g0.standard_normal(320).astype(F32)
+        lab0 = g0.integers(0, 10, 32).astype(np.uint32)
+        one0 = np.ones(32, F32)
+
+        def bn():
+            m = o.batch_mean(*d0, x0)
+            v = o.batch_var(*d0, 1e-5, x0, m)
+            o.batch_norm(*d0, x0, m, v)
+            dx = o.batch_norm_bwd(*d0, dy0, v)
+            dm = o.batch_norm_bwd_mean(*d0, dy0, v)
+            dv = o.batch_norm_bwd_var(*d0, dy0, x0, m, v)
+            dx = o.batch_var_bwd(*d0, dv, x0, m, dx_in=dx)
+            dm = o.batch_var_bwd_mean(*d0, dv, x0, m, dmean_in=dm)
+            o.batch_mean_bwd(*d0, dm, dx_in=dx)
+
+        def sm():
+            pr = o.softmax(10, 32, lg0)
+            o.softmax_cat_nll(10, 32, pr, lab0)
+            o.softmax_cat_nll_bwd(10, 32, one0, pr, lab0)
+
+        res = {}
+        for name, fn, reps in (("bn_fwd_bwd_cfg0", bn, 40), ("softmax_nll_cfg0", sm, 400)):
+            fn()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            res[name] = round((time.perf_counter() - t0) / reps * 1e6, 1)
+        return res
+
+    cfg0_one, cfg0_all = config0(1), config0(threads)
+    o.set_threads(threads)
+
     # repeat the sample until about 1.5 s of wall time on `threads` cores (~20-30 core-seconds), at most 16 passes
     passes = 0
     while passes < 16 and (passes == 0 or total_s < 1.5):
@@ -723,6 +810,10 @@ def cpu_baseline():
         "parts_gbps": {k: round(b / s / 1e9, 3) for k, (b, s) in parts.items()},
         "seconds": round(total_s, 2),
         "passes": passes,
+        "config0_us_per_pass": {k: {"cpu_us_1_thread": cfg0_one[k], f"cpu_us_{threads}_threads": cfg0_all[k]} for k in cfg0_one},
+        "config0_note": "BASELINE configs[0] (BN fwd+bwd [32,16,28,28], nine launches; softmax + NLL + backward [32,10], "
+                        "three launches) through the same fp32 restatement, called from Python (each call carries a few "
+                        "microseconds of ctypes overhead); the GPU figures for the same launches are small_shapes.*",
     }
 
 
@@ -731,6 +822,9 @@ def main():
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this build measures one GPU; --gpus above 1 is not supported\n")
         sys.exit(2)
+    if args.source_fingerprints:
+        print(json.dumps(source_fingerprints()), flush=True)
+        return
     import torch
 
     from anode_amd import gpu
@@ -838,16 +932,23 @@ def main():
         "frac": round(dom.alg_bytes / dom_s / 1e9 / HBM_PEAK_GBPS, 4),
         "alg_bytes_per_launch": dom.alg_bytes,
         "avg_launch_us": round(dom_s * 1e6, 2),
-        "traffic": MEASURED_TRAFFIC.get((dom.symbol, dom.group)),
         "traffic_source": TRAFFIC_SOURCE,
     }
+    fingerprints = source_fingerprints()
+    roofline["traffic"], note = measured_traffic(dom.symbol, dom.group, fingerprints)
+    if note:
+        roofline["traffic_note"] = note
+        sys.stderr.write(f"bench.py: roofline.traffic: {note}\n")
     # the same counters for the dominant kernel of every config (bytes per launch; ratio to the algorithmic bytes)
     traffic_by_kernel = []
     for l in launches:
-        t = MEASURED_TRAFFIC.get((l.symbol, l.group))
+        t, note = measured_traffic(l.symbol, l.group, fingerprints)
         if t is not None:
             traffic_by_kernel.append({"group": l.group, "symbol": l.symbol.replace("anode_gpu_", ""),
                                       "alg_bytes": l.alg_bytes, "traffic": t, "ratio": round(t / l.alg_bytes, 3)})
+        elif note:
+            traffic_by_kernel.append({"group": l.group, "symbol": l.symbol.replace("anode_gpu_", ""),
+                                      "alg_bytes": l.alg_bytes, "traffic": None, "note": note})
 
     groups = {}
     for l, t in zip(launches, med):
@@ -993,7 +1094,35 @@ def main():
             out["cpu_baseline"] = cpu_baseline()
         except Exception as e:  # noqa: BLE001
             out["cpu_baseline"] = {"error": repr(e)}
+    cb = out.get("cpu_baseline", {})
+    if isinstance(out.get("small_shapes"), dict) and "config0_us_per_pass" in cb:
+        for k, v in cb["config0_us_per_pass"].items():
+            if k in out["small_shapes"]:
+                out["small_shapes"][k]["cpu_us"] = v
+    out["targets"] = targets_block(breakdown, fused_model)
     print(json.dumps(out), flush=True)
+
+
+def targets_block(breakdown, fused_model):
+    """north_star's bar, machine-readable: every composite with its byte model and whether it sustains 70 % of the
+    8 TB/s HBM peak.  Launch-bound composites (config 3a: 1 MB arrays) are listed and flagged as such."""
+    notes = {
+        "softmax_cfg3a": "launch-bound: 1 MB arrays, 0.26 us at peak",
+        "fused_softmax_cfg3a": "launch-bound: 1 MB arrays",
+        "fused_softmax_fwd_bwd_cfg3a": "launch-bound: 1 MB arrays",
+        "softmax_cfg3b": "the reference ABI splits softmax and the label gather: with uniformly random labels the gather "
+                         "must touch 86 % of the probability tensor's 128-byte lines for 4 bytes per pixel (5.8 x its "
+                         "byte model), which holds this composite under 70 %; fused_softmax_fwd_cfg3b and "
+                         "fused_softmax_fwd_bwd_cfg3b are the same work without the gather",
+    }
+    out = {}
+    for model, table in (("abi", breakdown), ("fused", fused_model)):
+        for k, v in table.items():
+            e = {"pct_of_peak": v["pct_of_peak"], "byte_model": model, "met_70": bool(v["pct_of_peak"] >= 70.0)}
+            if k in notes:
+                e["note"] = notes[k]
+            out[k] = e
+    return out
 
 
 if __name__ == "__main__":
