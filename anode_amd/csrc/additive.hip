@@ -32,8 +32,8 @@ __device__ inline uint32_t quantize_one(float x, float lo, float scale) {
 // packs each to a dword, and the wave gathers the dwords through LDS so that each lane stores 16 consecutive bytes:
 // four 1 KiB loads and one 1 KiB store per wave, all contiguous, all four loads of a thread in flight together (the
 // input is read once, hence non-temporal).  One tile per workgroup, 4096 elements.  Measured 34.5 us at
-// [256,3,224,224] (57 us with one 16-byte load and one 4-byte store per thread).  `head` elements (0 to 15) come
-// first, one per thread of workgroup 0, so that the 16-byte stores lie on 16-byte boundaries wherever y lies; x is
+// [256,3,224,224] (57 us with one 16-byte load and one 4-byte store per thread).  `head` elements (0 to 127) come
+// first, one per thread of workgroup 0, so that the stores start on a 128-byte line wherever y lies; x is
 // read where it lies.
 __global__ __launch_bounds__(kBlock) void quantize_u8x16_kernel(uint32_t head, uint32_t n_groups, uint32_t tail,
                                                                 float lo, float scale, const float *__restrict__ x_,
@@ -110,8 +110,8 @@ struct FlatMultMap {
 // u8 codes -> per-channel affine f32: y = fma(scale[b], float(q), shift[b]).  One 16-byte load of 16 codes per
 // lane, the wave's dwords re-dealt through LDS (see wave_deal_dwords), each lane converts the four dwords it is
 // dealt; the channel of a group's first code is found by exact division, then advanced incrementally.  One tile per
-// workgroup, 4096 codes.  `head` elements (0 to 3) come first, one per thread of workgroup 0, so that the groups
-// of y start on a 16-byte boundary wherever y lies; the codes are read where they lie.
+// workgroup, 4096 codes.  `head` elements (0 to 31) come first, one per thread of workgroup 0, so that the groups
+// of y start on a 128-byte line wherever y lies; the codes are read where they lie.
 template <int NT>
 __global__ __launch_bounds__(kBlock) void bcast_dequantize_u8x16_kernel(uint32_t head, uint32_t n_dwords, uint32_t tail,
                                                                         FastDiv div_s, FastDiv div_c,
@@ -391,7 +391,7 @@ void launch_quantize(const char *symbol, uint32_t len, float lo, float hi, const
   if (len == 0) return;
   const float scale = (hi - lo) / 255.0f;
   hipStream_t s = as_stream(stream);
-  uint32_t head = uint32_t((16u - (reinterpret_cast<uintptr_t>(y) & 15u)) & 15u);  // bytes = elements of y
+  uint32_t head = uint32_t((128u - (reinterpret_cast<uintptr_t>(y) & 127u)) & 127u);  // bytes = elements of y
   if (head > len) head = len;
   const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
   const uint32_t blocks = (groups + kBlock * 4 - 1) / (kBlock * 4);
@@ -457,7 +457,7 @@ ANODE_EXPORT void anode_gpu_bcast_dequantize_u8_I1b_I2abc_Oabc_packed_f32(uint32
   if (len == 0) return;
   hipStream_t s = as_stream(stream);
   const FastDiv div_s(inner_dim), div_c(bcast_dim);
-  const uint32_t head = head_to_align16(y, len);
+  const uint32_t head = head_to_align_line(y, len);
   const uint32_t dwords = (len - head) / 4, tail = (len - head) % 4;
   const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
   with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal) & kNtStore, [&](auto policy) {

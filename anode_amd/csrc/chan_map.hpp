@@ -8,8 +8,8 @@
 // group, reloading the per-channel parameters only when a channel boundary is
 // crossed.  This keeps full 16-byte accesses for every S, including S that is
 // not a multiple of 4 (7x7 feature maps) and S == 1, and for arrays that start
-// at any element (a head of up to three elements is peeled so that the stores
-// lie on 16-byte boundaries; the inputs are read where they lie).
+// at any element (a head of up to 31 elements is peeled so that the stores
+// start on a 128-byte line; the inputs are read where they lie).
 #pragma once
 
 #include "common.hpp"
@@ -53,8 +53,8 @@ __device__ inline float chan_map_apply(const Op &op, const P &p, float x, float 
 // PAIR selects how a group that crosses a channel boundary gets its second parameter set: fetched up front beside
 // the first (channels of a few dozen elements, where a quarter of the groups cross), or on demand while walking
 // the group (long channels, where almost none does and the extra fetch and selects only cost issue slots).
-// `head` single elements (0 to 3) come before the groups, `tail` after them, both handled by workgroup 0: the
-// host picks head so that the groups of `out_` start on a 16-byte boundary wherever the array lies; the inputs are
+// `head` single elements (0 to 31) come before the groups, `tail` after them, both handled by workgroup 0: the
+// host picks head so that the groups of `out_` start on a 128-byte line wherever the array lies; the inputs are
 // read where they lie (4-byte aligned 16-byte loads).
 template <int NIN, bool ACC, int NT, bool PAIR, typename Op>
 __global__ __launch_bounds__(kBlock) void chan_map_kernel(uint32_t head, uint32_t n_groups, uint32_t tail,
@@ -217,7 +217,7 @@ void launch_chan_map(const char *symbol, uint32_t S, uint32_t C, uint32_t N, Op 
           S, N, uint32_t(threads), div_gpp, div_s, op, a, b, c, out);
     });
   } else {
-    const uint32_t head = head_to_align16(out, len);
+    const uint32_t head = head_to_align_line(out, len);
     const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
     const bool pair = S >= 4 && S < 4096;
     with_stream_policy(nt, [&](auto policy) {

@@ -113,8 +113,8 @@ __device__ inline uint32_t xcd_contiguous(uint32_t i, uint32_t n) {
 // arrays of the ABI are packed views that may start at any element, and a 16-byte access at such an address is the
 // same single instruction.  Measured on 822 MB arrays: a copy whose loads lie 4 bytes off a 16-byte boundary runs at
 // 6.55 TB/s against 6.65 aligned; streaming STORES off a boundary cost 15 % (5.6 TB/s: a wave's store then covers
-// parts of nine 128-byte lines instead of eight whole ones), so the maps peel a head of up to three elements to put
-// their stores on 16-byte boundaries and leave only the loads where they lie.
+// parts of nine 128-byte lines instead of eight whole ones), so the maps peel a head of up to 31 elements to start
+// their stores on a 128-byte line and leave only the loads where they lie.
 template <int NT, int ALIGN = 4, typename V>
 __device__ inline V load_stream(const V *p) {
   typedef V VU __attribute__((aligned(ALIGN)));
@@ -145,11 +145,24 @@ __device__ inline void store_stream(V *p, V v) {
   }
 }
 
-// Elements to peel off the front of an array of `len` 4-byte elements so that what follows starts on a 16-byte
-// boundary (0 to 3, never more than len).
-static inline uint32_t head_to_align16(const void *p, uint32_t len) {
-  const uint32_t h = uint32_t((16u - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u) / 4u;
+// Elements to peel off the front of an array of `len` 4-byte elements so that what follows starts on a 128-byte
+// line (0 to 31, never more than len).  Streaming stores want more than 16-byte alignment: a wave's store of 1 KiB
+// that starts 16 bytes into a 64-byte block leaves a partly written block at either end, and such stores, which
+// are written through, cost 12-15 % of the bandwidth (255 -> 292 us for batch_norm at [256,64,112,112]); starting
+// on a 64-byte boundary is enough, a whole line is as cheap to reach.
+static inline uint32_t head_to_align_line(const void *p, uint32_t len) {
+  const uint32_t h = uint32_t((128u - (reinterpret_cast<uintptr_t>(p) & 127u)) & 127u) / 4u;
   return h < len ? h : len;
+}
+
+// The streaming policy for kernels that cannot choose where their stores start (rows and planes lie where the
+// shape puts them): streaming stores only where every output array starts on a 64-byte boundary; otherwise the
+// default policy, whose stores are merged in the L2 before they leave ([8,19,512,1024] softmax one element past a
+// boundary: 161 us with streaming stores, 131 us without; 115 us on a boundary).
+static inline int policy_for_outputs(int nt, const void *out0, const void *out1 = nullptr) {
+  if ((reinterpret_cast<uintptr_t>(out0) & 63u) != 0) return 0;
+  if (out1 != nullptr && (reinterpret_cast<uintptr_t>(out1) & 63u) != 0) return 0;
+  return nt;
 }
 
 // Re-dealing a wave's dwords through LDS, for kernels whose narrow side would otherwise move 4 bytes per lane.

@@ -4,8 +4,8 @@
 //
 // Data path: every lane moves 16 bytes per access (global_load/store_dwordx4) and
 // consecutive lanes touch consecutive 16-byte groups.  Arrays may start at any
-// element: up to three head elements are peeled so that the stores lie on
-// 16-byte boundaries, and the loads are issued where the inputs lie.  All maps
+// element: up to 31 head elements are peeled so that the stores start on a
+// 128-byte line, and the loads are issued where the inputs lie.  All maps
 // read an element before writing the same index, so an output that aliases an
 // input at equal index is safe.
 #include "common.hpp"
@@ -79,7 +79,7 @@ __device__ inline f32x4 apply_vec(const Op &op, f32x4 a, f32x4 b) {
 }
 
 // `head` single elements, then n_groups groups of four, then `tail` single elements; the single elements are
-// handled by workgroup 0.  The host picks head so that the groups of `out_` start on a 16-byte boundary; the inputs
+// handled by workgroup 0.  The host picks head so that the groups of `out_` start on a 128-byte line; the inputs
 // are read where they lie (4-byte aligned 16-byte loads).
 template <int NIN, int NT, typename Op>
 __global__ __launch_bounds__(kBlock) void flat_map_kernel(uint32_t head, uint32_t n_groups, uint32_t tail, Op op,
@@ -113,7 +113,7 @@ void launch_flat_map(const char *symbol, uint32_t len, Op op, const float *a, co
   const Tuning &t = tuning();
   hipStream_t s = as_stream(stream);
   const int nt = stream_policy(size_t(len) * sizeof(float), t.nontemporal);
-  const uint32_t head = head_to_align16(out, len);
+  const uint32_t head = head_to_align_line(out, len);
   const uint32_t groups = (len - head) / 4, tail = (len - head) % 4;
   with_stream_policy(nt, [&](auto policy) {
     flat_map_kernel<NIN, decltype(policy)::value, Op>
@@ -140,8 +140,8 @@ struct DequantizeOp {
 // Each lane loads 16 codes in one access, the wave re-deals the dwords through LDS, and each lane converts the
 // four dwords it is dealt, so that every load (1 KiB) and every store (four of 1 KiB) of the wave is contiguous.
 // One tile per workgroup, 4096 codes.  Measured 34.7 us against 35.8 us for a form with one dword per lane at
-// [256,3,224,224].  `head` elements (0 to 3) come first, one per thread of workgroup 0, so that the groups of y
-// start on a 16-byte boundary wherever y lies; the codes are read where they lie (byte-aligned 16-byte loads).
+// [256,3,224,224].  `head` elements (0 to 31) come first, one per thread of workgroup 0, so that the groups of y
+// start on a 128-byte line wherever y lies; the codes are read where they lie (byte-aligned 16-byte loads).
 template <int NT, typename Op>
 __global__ __launch_bounds__(kBlock) void widen_u8x16_kernel(uint32_t head, uint32_t n_dwords, uint32_t tail, Op op,
                                                              const uint8_t *__restrict__ x_,
@@ -187,7 +187,7 @@ void launch_widen_u8(const char *symbol, uint32_t len, Op op, const uint8_t *x, 
   if (len == 0) return;
   const Tuning &t = tuning();
   hipStream_t s = as_stream(stream);
-  const uint32_t head = head_to_align16(y, len);
+  const uint32_t head = head_to_align_line(y, len);
   const uint32_t dwords = (len - head) / 4, tail = (len - head) % 4;
   const uint32_t blocks = (dwords + kBlock * 4 - 1) / (kBlock * 4);
   // the policy looks at the output, which is four times the input

@@ -682,7 +682,8 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
   // only runs again when the row count exceeds the grid limit
   const uint32_t max_blocks = 1u << 24;
   constexpr uint32_t kWavesPerBlock = kBlock / kWave;
-  const int nt = stream_policy(size_t(K) * R * sizeof(float), tuning().nontemporal);  // logits in, probabilities out: both streamed
+  // logits in, probabilities out: both streamed (streaming stores only for outputs that start on 64-byte boundaries)
+  const int nt = policy_for_outputs(stream_policy(size_t(K) * R * sizeof(float), tuning().nontemporal), y, nl.dx);
   if (K <= 224 || (K <= 256 && K % 16u != 0)) {
     // 1, 2, 4 or 8 lanes per row, at most 32 values per lane; the tile of 256 / G rows is at most 32 KiB.
     // The kernel is built for 4, 8, 16, 20, 24, 28 or 32 values per lane: the registers of a lane's array are what
@@ -1469,7 +1470,9 @@ void launch_softmax_nd_reg(uint32_t P, uint32_t C, uint32_t N, const float *x, f
   // keep the default policy unless they are far larger than the last-level cache
   const size_t bytes = size_t(P) * C * N * sizeof(float);
   if (PixVec<V>::W == 4) {
-    with_stream_policy(stream_policy(bytes, tuning().nontemporal), [&](auto policy) {
+    // (streaming stores only where every plane of the outputs starts on a 64-byte boundary)
+    const int nt = (P % 16u == 0) ? policy_for_outputs(stream_policy(bytes, tuning().nontemporal), y, dx) : 0;
+    with_stream_policy(nt, [&](auto policy) {
       launch_softmax_nd_reg_nt<V, NLL, decltype(policy)::value, BWD>(P, C, N, x, y, cat, nll, s, dy, dx);
     });
   } else {
@@ -1641,7 +1644,7 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
   const size_t lds_bytes = size_t(SB) * slab * sizeof(float);
   const FastDiv div_p(P), div_c(C);
   // logits in, probabilities (and the gradient) out: all streamed
-  const int nt = stream_policy(size_t(slab) * N * sizeof(float), tuning().nontemporal);
+  const int nt = policy_for_outputs(stream_policy(size_t(slab) * N * sizeof(float), tuning().nontemporal), y, dx);
   with_stream_policy(nt, [&](auto policy) {
     softmax_nd_tile_kernel<NLL, BWD, decltype(policy)::value>
         <<<blocks, kBlock, lds_bytes, s>>>(P, C, N, SB, div_p, div_c, vec, ignore ? 1u : 0u, x, y, cat, nll, dy, dx);
@@ -1849,7 +1852,7 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
   const FastDiv div_tps(ct.tiles_per_sample), div_tp(ct.TP);
   const uint32_t xcd = P >= 1024 ? 1u : 0u;
   // logits in, probabilities (and the gradient) out: all streamed
-  const int nt = stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal);
+  const int nt = policy_for_outputs(stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal), y, dx);
   with_stream_policy(nt, [&](auto policy) {
     softmax_nd_coltile_kernel<NLL, BWD, decltype(policy)::value><<<blocks, kBlock, lds_bytes, s>>>(
         P, C, ct.TP, ct.L, total_tiles, div_tps, div_tp, ignore ? 1u : 0u, xcd, x, y, cat, nll, dy, dx);
@@ -1997,7 +2000,7 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
   if (vec && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
     const uint32_t total_groups = len / 4u;
     const FastDiv div_gpp(P / 4u), div_c(C);
-    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
+    with_stream_policy(policy_for_outputs(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), dx), [&](auto policy) {
       softmax_nd_cat_nll_bwd_flat_kernel<ACC, decltype(policy)::value>
           <<<stream_grid(total_groups, 1), kBlock, 0, s>>>(P, C, total_groups, div_gpp, div_c, ignore ? 1u : 0u, dy, prob,
                                                           cat, dx);
@@ -2006,7 +2009,8 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
     PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);
     pg.xcd = (tuning().nd_xcd_mask & 2) ? 1u : 0u;
     const dim3 grid = nd_bwd_grid(pg.total_groups, C, chunk);
-    with_stream_policy(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), [&](auto policy) {
+    const int nt = (P % 16u == 0) ? policy_for_outputs(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), dx) : 0;
+    with_stream_policy(nt, [&](auto policy) {
       softmax_nd_cat_nll_bwd_kernel<f32x4, ACC, decltype(policy)::value>
           <<<grid, kBlock, 0, s>>>(pg, dy, prob, cat, dx, chunk);
     });

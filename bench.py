@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--shape-sweep", action="store_true",
                     help="instead of the benchmark: batch-norm pieces over S x C, row softmax over K and channel-axis "
                          "softmax over C x P, each on ~256 MB arrays, one JSON line (where the tilings switch)")
+    ap.add_argument("--offset-views", action="store_true",
+                    help="instead of the benchmark: the configs' dominant entry points with arrays on 16-byte "
+                         "boundaries, one element past them, and 1, 2, 3 elements past them, one JSON line")
     ap.add_argument("--source-fingerprints", action="store_true",
                     help="print the fingerprints of the kernel sources behind the measured-traffic table and exit")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -590,6 +593,100 @@ def all_symbols(torch, gpu):
     return rows
 
 
+def offset_views(torch, gpu):
+    """Arrays that are views starting at any element (as_dptr() on a view): the entry points named below at the
+    configs' shapes with every array on a 16-byte boundary, with every array one element past one (the same view of
+    sibling arrays), and with the arrays 1, 2 and 3 elements past one (views that lie differently).  Launches of the
+    three placements are made in rotation; median of 20."""
+    E = lambda n, dt=torch.float32: torch.empty(n + 8, device="cuda", dtype=dt)  # noqa: E731
+    placements = {"aligned": (0, 0, 0, 0), "all_plus_1": (1, 1, 1, 1), "plus_1_2_3": (1, 2, 3, 1)}
+    cases = []
+
+    def case(name, shape, nbytes, make):
+        cases.append((name, shape, nbytes, make))
+
+    def view(t, off, n):
+        return t[off:off + n]
+
+    for tag, (S, C, N) in (("cfg2a [256,64,112,112]", (12544, 64, 256)), ("cfg2b [256,2048,7,7]", (49, 2048, 256)),
+                           ("cfg4 [2,32,128,128,128]", (128 ** 3, 32, 2))):
+        n = S * C * N
+        x, dy, y = torch.randn(n + 8, device="cuda"), torch.randn(n + 8, device="cuda"), E(n)
+        m, v, dv, o = torch.randn(C + 8, device="cuda"), torch.rand(C + 8, device="cuda") + 0.5, torch.randn(C + 8, device="cuda"), E(C)
+        d = (S, C, N)
+        case("batch_mean_3d1_packed_f32", tag, 4 * n,
+             lambda a, b, c, e, d=d, x=x, o=o, n=n, C=C: ("anode_gpu_batch_mean_3d1_packed_f32", (*d, view(x, a, n), view(o, e, C))))
+        case("batch_norm_bwd_var_3d1_packed_f32", tag, 8 * n,
+             lambda a, b, c, e, d=d, x=x, dy=dy, m=m, v=v, o=o, n=n, C=C:
+             ("anode_gpu_batch_norm_bwd_var_3d1_packed_f32", (*d, view(dy, a, n), view(x, b, n), view(m, e, C), view(v, e, C), view(o, e, C))))
+        case("batch_norm_3d1_packed_f32", tag, 8 * n,
+             lambda a, b, c, e, d=d, x=x, y=y, m=m, v=v, n=n, C=C:
+             ("anode_gpu_batch_norm_3d1_packed_f32", (*d, view(x, a, n), view(m, e, C), view(v, e, C), view(y, b, n))))
+        case("batch_var_bwd_3d1_packed_accumulate_f32", tag, 12 * n,
+             lambda a, b, c, e, d=d, x=x, y=y, m=m, dv=dv, n=n, C=C:
+             ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", (*d, view(dv, e, C), view(x, a, n), view(m, e, C), view(y, b, n))))
+        if tag.startswith("cfg4"):
+            case("positive_clip_flat_map_f32", tag, 8 * n,
+                 lambda a, b, c, e, x=x, y=y, n=n: ("anode_gpu_positive_clip_flat_map_f32", (n, view(x, a, n), view(y, b, n))))
+            case("positive_clip_flat_map_bwd_f32", tag, 12 * n,
+                 lambda a, b, c, e, x=x, y=y, dy=dy, n=n:
+                 ("anode_gpu_positive_clip_flat_map_bwd_f32", (n, view(dy, a, n), view(x, b, n), view(y, c, n))))
+    P, C, N = 512 * 1024, 19, 8
+    n = P * C * N
+    x, p, dx = torch.randn(n + 8, device="cuda"), E(n), E(n)
+    lab = torch.randint(0, C, (P * N + 8,), device="cuda", dtype=torch.int32)
+    dy, nll = torch.ones(P * N + 8, device="cuda"), E(P * N)
+    tag = "cfg3b [8,19,512,1024]"
+    case("softmax_nd_packed_f32", tag, 8 * n,
+         lambda a, b, c, e: ("anode_gpu_softmax_nd_packed_f32", (P, C, N, view(x, a, n), view(p, b, n))))
+    case("softmax_nd_cat_nll_bwd_packed_f32", tag, 8 * n + 8 * P * N,
+         lambda a, b, c, e: ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32",
+                             (P, C, N, view(dy, e, P * N), view(p, a, n), view(lab, c, P * N), view(dx, b, n))))
+    case("softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", tag, 12 * n + 12 * P * N,
+         lambda a, b, c, e: ("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32",
+                             (P, C, N, view(x, a, n), view(lab, c, P * N), view(dy, e, P * N), view(p, b, n),
+                              view(nll, e, P * N), view(dx, c, n))))
+    K, R = 1000, 65536
+    case("softmax_packed_deterministic_f32", "[65536,1000]", 8 * K * R,
+         lambda a, b, c, e: ("anode_gpu_softmax_packed_deterministic_f32", (K, R, view(x, a, K * R), view(p, b, K * R))))
+    nq = 256 * 3 * 224 * 224
+    q = torch.randint(0, 256, (nq + 32,), device="cuda", dtype=torch.uint8)
+    zq = torch.empty(nq + 32, device="cuda", dtype=torch.uint8)
+    tag = "cfg1 [256,3,224,224]"
+    case("dequantize_u8_packed_f32", tag, 5 * nq,
+         lambda a, b, c, e: ("anode_gpu_dequantize_u8_packed_f32", (nq, 0.0, 1.0, view(q, a, nq), view(p, b, nq))))
+    case("quantize_u8_packed_f32", tag, 5 * nq,
+         lambda a, b, c, e: ("anode_gpu_quantize_u8_packed_f32", (nq, -4.0, 4.0, view(x, a, nq), view(zq, b, nq))))
+
+    rows = []
+    for name, shape, nbytes, make in cases:
+        calls = {k: make(*offs) for k, offs in placements.items()}
+        for sym, args in calls.values():
+            gpu.call(sym, *args)
+        torch.cuda.synchronize()
+        times = {k: [] for k in calls}
+        for _ in range(20):
+            evs = {}
+            for k, (sym, args) in calls.items():
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                gpu.call(sym, *args)
+                b.record()
+                evs[k] = (a, b)
+            torch.cuda.synchronize()
+            for k, (a, b) in evs.items():
+                times[k].append(a.elapsed_time(b) * 1e-3)
+        assert gpu.take_last_error() == 0
+        row = {"symbol": name, "shape": shape}
+        for k, ts in times.items():
+            t = sorted(ts)[len(ts) // 2]
+            row[k] = {"us": round(t * 1e6, 1), "gbps": round(nbytes / t / 1e9, 1)}
+        row["all_plus_1_vs_aligned"] = round(row["all_plus_1"]["gbps"] / row["aligned"]["gbps"], 3)
+        row["plus_1_2_3_vs_aligned"] = round(row["plus_1_2_3"]["gbps"] / row["aligned"]["gbps"], 3)
+        rows.append(row)
+    return rows
+
+
 def graph_replay(torch, run_step, steps, step_bytes):
     """The same step captured once as a HIP graph and replayed: what the launch gaps cost (reported beside `value`,
     which stays the plainly launched figure)."""
@@ -841,6 +938,9 @@ def main():
         return
     if args.all_symbols:
         print(json.dumps({"all_symbols": all_symbols(torch, gpu), "peak_gbps": HBM_PEAK_GBPS}), flush=True)
+        return
+    if args.offset_views:
+        print(json.dumps({"offset_views": offset_views(torch, gpu), "peak_gbps": HBM_PEAK_GBPS}), flush=True)
         return
     only = set(filter(None, args.only.split(",")))
     launches, fused = build_workload(torch, only, args.copy_calibration)
