@@ -394,6 +394,35 @@ def stream_probe(torch, gpu):
         "softmax_nd (all planes, then store)": rate(
             lambda i: gpu.call("anode_gpu_softmax_nd_packed_f32", P, Cc, Nn, *sets[i % 3]), 8 * m),
     }
+    del sets
+    torch.cuda.empty_cache()
+
+    def one(fn):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e-3
+
+    # What the launch before it does to a kernel: dequantize of u8 [256,3,224,224] (38.5 MB in, 154 MB out) right
+    # after a reader (batch_mean over 822 MB) and right after a writer (copy of 822 MB), library defaults.
+    nq = 256 * 3 * 224 * 224
+    q = torch.randint(0, 256, (nq,), device="cuda", dtype=torch.uint8)
+    yq = torch.empty(nq, device="cuda")
+    Sb, Cb, Nb = 12544, 64, 256
+    big = torch.randn(Sb * Cb * Nb, device="cuda")
+    bigdst = torch.empty(Sb * Cb * Nb, device="cuda")
+    mean = torch.empty(Cb, device="cuda")
+    after_reader, after_writer = [], []
+    for _ in range(8):
+        gpu.call("anode_gpu_batch_mean_3d1_packed_f32", Sb, Cb, Nb, big, mean)
+        after_reader.append(one(lambda: gpu.call("anode_gpu_dequantize_u8_packed_f32", nq, 0.0, 1.0, q, yq)))
+        gpu.call("anode_gpu_copy_flat_map_f32", big.numel(), big, bigdst)
+        after_writer.append(one(lambda: gpu.call("anode_gpu_dequantize_u8_packed_f32", nq, 0.0, 1.0, q, yq)))
+    med = lambda t: sorted(t[1:])[len(t[1:]) // 2]  # noqa: E731
+    out["dequantize_cfg1_us"] = {"after_a_reader_of_822MB": round(med(after_reader) * 1e6, 1),
+                                 "after_a_writer_of_822MB": round(med(after_writer) * 1e6, 1)}
     return out
 
 
