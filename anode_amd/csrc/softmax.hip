@@ -82,6 +82,7 @@ __device__ inline float exp_nonpos(float d) {
   const float e = __builtin_amdgcn_exp2f(t);
   return fmaf(e, r * kLn2, e);
 }
+__device__ inline f32x4 vexp4(f32x4 a) { return f32x4{exp_nonpos(a.x), exp_nonpos(a.y), exp_nonpos(a.z), exp_nonpos(a.w)}; }
 // Marks the point from which a loaded value is known to have arrived.  The streaming stores are inline assembly,
 // which the compiler's wait-count bookkeeping does not see: where the first use of an earlier load sits in a
 // conditional block after such stores, the wait it inserts there (for "the load") also waits for every store
@@ -409,6 +410,112 @@ __global__ __launch_bounds__(THREADS) void softmax_row_blockreg_kernel(uint32_t 
   }
 }
 
+// Rows of up to 64 * THREADS classes in whole 16-byte groups, read once: one workgroup per row, the row's first half
+// (the first 8 * THREADS slots) in LDS and its second half in registers, 32 values per thread each.  512 threads
+// hold 32768 classes in 64 KB of LDS, so two workgroups fit a CU and one loads while the other reduces or stores
+// (the register-only kernel above needs 1024 threads for such rows, one workgroup per CU, whose CU idles between its
+// phases); 1024 threads hold 65536 classes in 128 KB of the CU's 160 KB, where the streaming kernel below keeps
+// 16384 values and reads the rest a second time.  A thread's 16 slots are taken in two batches of eight 16-byte
+// loads; the held half goes to LDS as it arrives, is read back for the sum of exponentials and once more for the
+// normalised values.  Slots are dealt as in the register kernel (a step of the workgroup covers an aligned run of
+// the array).  The row's sum is the workgroup sum of the threads' sums, each added in slot order, LDS half first.
+template <int THREADS, int NT>
+__global__ __launch_bounds__(THREADS) void softmax_row_reglds_kernel(uint32_t K, uint32_t R,
+                                                                    const float *__restrict__ x,
+                                                                    float *__restrict__ y, RowNll nl) {
+  constexpr int NGH = 8;                           // groups per thread in each half
+  constexpr uint32_t kSlots = 2u * NGH * THREADS;  // a power of two
+  extern __shared__ __align__(16) float held_row[];  // NGH * THREADS groups of 16 bytes
+  f32x4 *held = reinterpret_cast<f32x4 *>(held_row);
+  __shared__ float lds[THREADS / kWave];
+  for (uint64_t r = blockIdx.x; r < R; r += gridDim.x) {
+    const float *xr = x + size_t(r) * K;
+    float *yr = y + size_t(r) * K;
+    float *dxr = (nl.on() && nl.dx != nullptr) ? nl.dx + size_t(r) * K : nullptr;
+    const uint32_t a = (uint32_t(r) * (K / 4u)) & 7u;  // the row's distance in groups from a 128-byte line of the array
+    auto kof = [&](int i) -> uint32_t {  // first class of slot i of this thread
+      const uint32_t slot = threadIdx.x + uint32_t(i) * uint32_t(THREADS);
+      return ((slot + kSlots - a) & (kSlots - 1u)) * 4u;
+    };
+    const uint32_t label = nl.on() ? nl.label(r) : 0u;
+    const float dyr = dxr != nullptr ? nl.dy[r] : 0.0f;
+    const f32x4 ninf = f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+    float m = kNegInf;
+    // first half: to LDS
+    {
+      f32x4 t[NGH];
+#pragma unroll
+      for (int i = 0; i < NGH; ++i) {
+        const uint32_t k = kof(i);
+        t[i] = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k)) : ninf;
+      }
+#pragma unroll
+      for (int i = 0; i < NGH; ++i) {
+        held[uint32_t(i) * THREADS + threadIdx.x] = t[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m = fmaxf(m, t[i][j]);
+      }
+    }
+    // second half: stays in registers
+    f32x4 v[NGH];
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {
+      const uint32_t k = kof(NGH + i);
+      v[i] = (k < K) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xr + k)) : ninf;
+    }
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) m = fmaxf(m, v[i][j]);
+    }
+    m = block_max<THREADS / kWave>(m, lds);
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {  // (a slot past the row's end holds -inf and adds exp(-inf - m) = 0, NaN only if m is)
+      const f32x4 t = held[uint32_t(i) * THREADS + threadIdx.x];
+      const bool in = kof(i) < K;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s += in ? exp_nonpos(t[j] - m) : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {
+      const bool in = kof(NGH + i) < K;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[i][j] = in ? exp_nonpos(v[i][j] - m) : 0.0f;
+        s += v[i][j];
+      }
+    }
+    s = block_sum<float, THREADS / kWave>(s, lds);
+    const float rs = 1.0f / s;  // one correctly rounded reciprocal per row
+    auto emit = [&](uint32_t k, f32x4 pr) {
+      if (nl.on()) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) nl.emit_nll(r, K, label, k + uint32_t(j), pr[j]);
+      }
+      store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), pr);
+      if (dxr != nullptr) {
+        store_stream<NT>(reinterpret_cast<f32x4 *>(dxr + k),
+                         f32x4{RowNll::grad(dyr, label, k, pr[0]), RowNll::grad(dyr, label, k + 1u, pr[1]),
+                               RowNll::grad(dyr, label, k + 2u, pr[2]), RowNll::grad(dyr, label, k + 3u, pr[3])});
+      }
+    };
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {
+      const uint32_t k = kof(NGH + i);
+      if (k < K) emit(k, v[i] * rs);
+    }
+#pragma unroll
+    for (int i = 0; i < NGH; ++i) {
+      const uint32_t k = kof(i);
+      if (k < K) {
+        const f32x4 t = held[uint32_t(i) * THREADS + threadIdx.x];
+        emit(k, vexp4(t - m) * rs);
+      }
+    }
+  }
+}
+
 // any K: workgroups of 512 threads, two to a CU, each walking rows.  A row is taken in batches of U groups of W
 // values per thread (a slot past the row's end reads the last group again and counts as -inf) and folded into a
 // running maximum and a running sum of exponentials about it; the next batch is requested before the current one
@@ -673,6 +780,22 @@ __global__ __launch_bounds__(kRowStreamThreads) __attribute__((amdgpu_waves_per_
   }
 }
 
+template <int THREADS, int NT>
+void launch_softmax_row_reglds(uint32_t blocks, uint32_t K, uint32_t R, const float *x, float *y, const RowNll &nl,
+                               hipStream_t s) {
+  constexpr size_t lds_bytes = size_t(8) * THREADS * 16;
+  // more than the 64 KB a kernel may take by default: raised once per device
+  static std::atomic<bool> raised[64];
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev >= 0 && dev < 64 && !raised[dev].load(std::memory_order_relaxed)) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&softmax_row_reglds_kernel<THREADS, NT>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    raised[dev].store(true, std::memory_order_relaxed);
+  }
+  softmax_row_reglds_kernel<THREADS, NT><<<blocks, THREADS, lds_bytes, s>>>(K, R, x, y, nl);
+}
+
 void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float *x, float *y,
                          CUstream_st *stream, RowNll nl = RowNll{nullptr, nullptr, false, nullptr, nullptr}) {
   (void)checked_len(K, R, 1, symbol);
@@ -801,15 +924,21 @@ void launch_softmax_rows(const char *symbol, uint32_t K, uint32_t R, const float
       } else {
         softmax_row_blockreg_kernel<32, false, 0, 512><<<blocks, 512, 0, s>>>(K, R, x, y, nl);
       }
-    } else if (K <= 32768) {
-      // workgroups of 1024 threads, 32 values each
-      if (vec) {
-        with_stream_policy(nt, [&](auto policy) {
-          softmax_row_blockreg_kernel<32, true, decltype(policy)::value, 1024><<<blocks, 1024, 0, s>>>(K, R, x, y, nl);
-        });
-      } else {
-        softmax_row_blockreg_kernel<32, false, 0, 1024><<<blocks, 1024, 0, s>>>(K, R, x, y, nl);
-      }
+    } else if (vec && K <= 32768 && (tuning().row_reglds & 1)) {
+      // workgroups of 512 threads, two to a CU: half of the row in LDS, half in registers ([2730, 24576] 4.8 -> 5.8
+      // TB/s, [2048, 32768] 4.9 -> 5.5 against 1024 threads with the whole row in registers, one workgroup per CU)
+      with_stream_policy(nt, [&](auto policy) { launch_softmax_row_reglds<512, decltype(policy)::value>(blocks, K, R, x, y, nl, s); });
+    } else if (vec && K <= 65536 && (tuning().row_reglds & 2)) {
+      // one workgroup of 1024 threads per CU: half of the row in 128 KB of LDS, half in registers; x is read once
+      // ([1335, 50256] 4.2 -> 4.6 TB/s, [1024, 65536] 4.65 -> 5.05, [2047, 32772] 4.1 -> 4.6 against the streaming
+      // kernel below; [1864, 36000] and [1677, 40000] 4.5 and 4.7 either way)
+      const uint32_t cus = uint32_t(device_cu_count());
+      with_stream_policy(nt, [&](auto policy) {
+        launch_softmax_row_reglds<1024, decltype(policy)::value>(R < cus ? R : cus, K, R, x, y, nl, s);
+      });
+    } else if (!vec && K <= 32768) {
+      // rows that are not whole 16-byte groups: workgroups of 1024 threads, 32 values each, 4-byte accesses
+      softmax_row_blockreg_kernel<32, false, 0, 1024><<<blocks, 1024, 0, s>>>(K, R, x, y, nl);
     } else {
       // two workgroups per CU, which walk their rows
       const uint32_t cus = 2u * uint32_t(device_cu_count());
