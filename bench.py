@@ -993,8 +993,11 @@ def main():
     assert gpu.take_last_error() == 0
 
     # untimed calibration pass: per-launch HIP-event durations for the breakdown
+    # (11 passes back to back, the first dropped: a launch made on an idle GPU, as the first launch after a
+    # synchronisation is, measures about 6 us more between its events than the same launch inside a sequence)
     per_launch = [[] for _ in launches]
-    for _ in range(10):
+    all_evs = []
+    for _ in range(11):
         evs = []
         for l in launches:
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -1002,7 +1005,9 @@ def main():
             gpu.call(l.symbol, *l.args)
             b.record()
             evs.append((a, b))
-        torch.cuda.synchronize()
+        all_evs.append(evs)
+    torch.cuda.synchronize()
+    for evs in all_evs[1:]:
         for i, (a, b) in enumerate(evs):
             per_launch[i].append(a.elapsed_time(b) * 1e-3)
     med = [sorted(t)[len(t) // 2] for t in per_launch]
@@ -1101,7 +1106,8 @@ def main():
             gpu.call(l.symbol, *l.args)
         torch.cuda.synchronize()
         ftimes = [[] for _ in fused]
-        for _ in range(10):
+        all_evs = []
+        for _ in range(11):  # back to back, the first pass dropped (see above)
             evs = []
             for l in fused:
                 a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -1109,7 +1115,9 @@ def main():
                 gpu.call(l.symbol, *l.args)
                 b.record()
                 evs.append((a, b))
-            torch.cuda.synchronize()
+            all_evs.append(evs)
+        torch.cuda.synchronize()
+        for evs in all_evs[1:]:
             for i, (a, b) in enumerate(evs):
                 ftimes[i].append(a.elapsed_time(b) * 1e-3)
         assert gpu.take_last_error() == 0

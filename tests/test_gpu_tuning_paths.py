@@ -26,6 +26,10 @@ PROFILES = {
     # to the kernel that gives a thread four pixels and walks their classes (the default only does so from 131073 on)
     "nd_backward_by_pixel_groups": {14: 0},
     "nd_backward_by_pixel_groups_nontemporal": {14: 0, 5: 0},
+    # knob 15: rows of 16385 to 65536 classes held half in LDS, half in registers; 0 sends them to the streaming kernel
+    "long_rows_streamed": {15: 0},
+    "long_rows_streamed_nontemporal": {15: 0, 5: 0},
+    "long_rows_half_in_lds_nontemporal": {5: 0},
 }
 
 
@@ -56,7 +60,7 @@ def test_flat_maps_under_tuning(tuned, oracle):
 
 
 def test_softmax_under_tuning(tuned, oracle):
-    for K, R in [(10, 4000), (1000, 256), (4096, 3), (40000, 1)]:
+    for K, R in [(10, 4000), (1000, 256), (4096, 3), (40000, 1), (16388, 3), (32768, 2), (65536, 2)]:
         for name in T_sm.ROW_ENTRY_POINTS:
             T_sm.test_softmax_rows(oracle, name, K, R)
     T_sm.test_softmax_cat_nll_and_bwd_rows(oracle, 1000, 256)
