@@ -601,17 +601,21 @@ def all_symbols(torch, gpu):
         gpu.call(sym, *args)
     torch.cuda.synchronize()
     times = [[] for _ in L]
-    for _ in range(50):
-        evs = []
-        for sym, _, args, _ in L:
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            gpu.call(sym, *args)
-            b.record()
-            evs.append((a, b))
+    for _ in range(5):  # five runs of eleven rotations back to back, the first rotation of each run dropped (it starts on an idle GPU)
+        runs = []
+        for _ in range(11):
+            evs = []
+            for sym, _, args, _ in L:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                gpu.call(sym, *args)
+                b.record()
+                evs.append((a, b))
+            runs.append(evs)
         torch.cuda.synchronize()
-        for i, (a, b) in enumerate(evs):
-            times[i].append(a.elapsed_time(b) * 1e-3)
+        for evs in runs[1:]:
+            for i, (a, b) in enumerate(evs):
+                times[i].append(a.elapsed_time(b) * 1e-3)
     assert gpu.take_last_error() == 0
     rows = []
     for (sym, shape, _, nbytes), ts in zip(L, times):
