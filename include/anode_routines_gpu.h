@@ -11,8 +11,10 @@
  *
  * Conventions shared by every entry point (reference: lib.h:27-39,
  * common.cuh:51-67, src/ops_gpu.rs:670-679):
- *   - all data pointers are DEVICE pointers to packed arrays; `cfg` is a HOST
- *     pointer, read during the call;
+ *   - all data pointers are DEVICE pointers to packed arrays; they need the
+ *     alignment of their element type and nothing more (views that start at
+ *     any element of an allocation run the same 16-byte kernels); `cfg` is a
+ *     HOST pointer, read during the call;
  *   - `stream` is the runtime's stream handle (a hipStream_t passed through the
  *     opaque struct CUstream_st*; NULL = the null stream);
  *   - the call enqueues work on `stream` and returns; nothing is reported;
@@ -244,9 +246,10 @@ void anode_gpu_batch_norm_bwd_apply_3d1_packed_f32(uint32_t dim0, uint32_t dim1,
 void anode_gpu_batch_norm_bwd_apply_3d1_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *dy, const float *x, const float *mean, const float *var, const float *dmean, const float *dvar, const float *mask, float *dx, ANODE_LAUNCH_TAIL);
 /* Row softmax and softmax_cat_nll in one pass over x (src/ops.rs:1172-1176 as one launch); writes the same softmax and
  * nll as anode_gpu_softmax_packed_*_f32 followed by anode_gpu_softmax_cat_nll_packed_f32 (NaN for a label >= dim0).
- * "The same" is to the bit where the arrays of the two calls lie alike: the order in which a row's exponentials are
- * added may depend on where x and the outputs start within a 128-byte line (16-byte or 4-byte accesses; for rows of
- * more than 32768 classes at element offsets, the place of the row in a line of the output). */
+ * "The same" is to the bit: the kernel, and with it the order in which a row's exponentials are added, follows the
+ * shape alone.  The one exception is rows of more than 32768 classes whose length is not a multiple of four: there
+ * the order depends on where a row starts within a 128-byte line of the output, so the two agree to the bit where
+ * the arrays of the two calls lie alike (as arrays handed out by an allocator do). */
 void anode_gpu_softmax_cat_nll_fused_packed_f32(uint32_t dim0, uint32_t dim1, const float *x, const uint32_t *cat_data, float *softmax, float *nll, ANODE_LAUNCH_TAIL);
 /* The same plus anode_gpu_softmax_cat_nll_bwd_packed_f32 in that launch, for a dy that is known before the forward
  * pass (e.g. ones for a summed loss): dx[k,i] = dy[i] * (softmax[k,i] - float(label[i]==k)). */

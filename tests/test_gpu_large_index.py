@@ -97,6 +97,38 @@ def test_softmax_nd_beyond_2_31(big):
     del p, sums
 
 
+def test_softmax_nd_samples_of_more_than_4_gib(big):
+    # Planes of 64 Mi pixels: a sample of 17 planes is 4.5 GB, so the byte offsets of a wave that crosses from one
+    # sample into the next (and of the odd lane's plane pitch) no longer fit 32 bits and the two-lane kernel takes
+    # its form with 64-bit lane offsets.  Two samples, the plain and the fused forward + backward entry points.
+    P, C, N = 1 << 26, 17, 1
+    n = P * C * N
+    assert n <= N_BIG
+    x = big[:n]
+    p = torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_packed_f32", P, C, N, x, p)
+    torch.cuda.synchronize()
+    xv, pv = x.view(C, P), p.view(C, P)
+    for lo in (0, P // 2 - 4096, P - 8192):                # float64 checks on slices of the pixels
+        ref = torch.softmax(xv[:, lo:lo + 8192].double(), dim=0)
+        assert bool(((pv[:, lo:lo + 8192].double() - ref).abs() <= 1e-5 * ref).all())
+    assert bool(((pv.sum(dim=0) - 1).abs() < 1e-5).all())
+    lab = torch.randint(0, C, (P * N,), device="cuda", dtype=torch.int32)
+    dy = torch.randn(P * N, device="cuda")
+    p2, nll, dx = torch.empty(n, device="cuda"), torch.empty(P * N, device="cuda"), torch.empty(n, device="cuda")
+    call("anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32", P, C, N, x, lab, dy, p2, nll, dx)
+    torch.cuda.synchronize()
+    assert torch.equal(p2, p)
+    picked = torch.gather(pv, 0, lab.long().unsqueeze(0)).squeeze(0)
+    assert torch.allclose(nll, -torch.log(picked), rtol=1e-5, atol=1e-6)
+    ks = torch.arange(C, device="cuda", dtype=torch.int32).view(C, 1)
+    for lo in (0, P - 8192):
+        sl = slice(lo, lo + 8192)
+        want = dy[sl].unsqueeze(0) * (pv[:, sl] - (lab[sl].unsqueeze(0) == ks).float())
+        assert torch.equal(dx.view(C, P)[:, sl], want)
+    del p, p2, nll, dx, picked
+
+
 def test_softmax_nd_backward_beyond_2_31(big):
     # planes of up to 131072 pixels: the backward pass walks the array flat, one 16-byte group of dx per thread
     P, C, N = 1 << 16, 19, 1725
