@@ -59,8 +59,10 @@ struct ReducePlan {
   uint32_t J;         // lane tiles: samples that the lanes of a workgroup take side by side; otherwise 0
 };
 
-// Host-side tiling decision; `ptrs_aligned` says whether every element array
-// is 16-byte aligned, `nin` how many element arrays the reduction reads.  Exposed (anode_gpu_plan_reduce) so that it can be
+// Host-side tiling decision; `ptrs_aligned` says whether the 16-byte tilings
+// may be taken (the launcher always says yes: loads only need 4-byte alignment;
+// the 4-byte tilings remain for the geometries that have no 16-byte form and
+// for the planner's tests), `nin` how many element arrays the reduction reads.  Exposed (anode_gpu_plan_reduce) so that it can be
 // checked without a device.
 ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligned, uint32_t wg_target, int nin);
 

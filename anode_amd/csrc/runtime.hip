@@ -179,7 +179,7 @@ ReducePlan plan_chan_reduce(uint32_t S, uint32_t C, uint32_t N, bool ptrs_aligne
     p.SB = S;
     p.n_stiles = 1;
     bool vec = ptrs_aligned && (uint64_t(C) * S) % 4 == 0;
-    // a tile that is not the whole channel axis must start on a 16-byte boundary: CB*S a multiple of 4
+    // a tile that is not the whole channel axis must start a whole number of 16-byte groups into the array: CB*S a multiple of 4
     const uint32_t unit = 4 / gcd_u32(S, 4);
     const uint32_t lane_cap = kBlock * (vec ? 4u : 1u);  // positions that one pass of a workgroup's lanes covers
     // (with 16-byte accesses a tile is either the whole channel axis or a multiple of `unit` channels: one of the

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_lds_kernel(uint32_t K, uin
     const uint32_t n = rows * K;
     const float *xt = x + r0 * K;
     float *yt = y + r0 * K;
-    // (the tile starts a multiple of 32 rows into an aligned array: 16-byte aligned)
+    // (the tile starts a multiple of 32 rows, hence a whole number of 16-byte groups, into the array)
     const uint32_t n4 = vec ? n / 4u : 0u;
     // the row's label and upstream gradient are requested together with the tile
     const uint64_t r = r0 + local;
@@ -235,8 +235,8 @@ uint32_t pick_row_rotation(uint32_t K, uint32_t log2g) {
   return best;
 }
 
-// Up to 64 * VPL columns (from 225 on, see the dispatch): one wave per row, VPL values per lane.  VEC: rows start on 16-byte boundaries (K a multiple
-// of 4, aligned arrays) and a lane owns groups of four consecutive classes; otherwise lane l owns k = l, l+64, ...
+// Up to 64 * VPL columns (from 225 on, see the dispatch): one wave per row, VPL values per lane.  VEC: rows are whole 16-byte groups (K a multiple
+// of 4) and a lane owns groups of four consecutive classes; otherwise lane l owns k = l, l+64, ...
 template <int VPL, bool VEC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, uint32_t R,
                                                                   const float *__restrict__ x,
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(kBlock) void softmax_row_wave_kernel(uint32_t K, ui
         }
         if (VEC) {
           store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
-          if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
+          if (nl.on() && nl.dx != nullptr) {
             store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
                              f32x4{RowNll::grad(dyr, label, k, v[i * W]), RowNll::grad(dyr, label, k + 1u, v[i * W + 1]),
                                    RowNll::grad(dyr, label, k + 2u, v[i * W + 2]),
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(THREADS) void softmax_row_blockreg_kernel(uint32_t 
         }
         if (VEC) {
           store_stream<NT>(reinterpret_cast<f32x4 *>(yr + k), f32x4{v[i * W], v[i * W + 1], v[i * W + 2], v[i * W + 3]});
-          if (nl.on() && nl.dx != nullptr) {  // the host checked that dx is 16-byte aligned as well
+          if (nl.on() && nl.dx != nullptr) {
             store_stream<NT>(reinterpret_cast<f32x4 *>(nl.dx + size_t(r) * K + k),
                              f32x4{RowNll::grad(dyr, label, k, v[i * W]), RowNll::grad(dyr, label, k + 1u, v[i * W + 1]),
                                    RowNll::grad(dyr, label, k + 2u, v[i * W + 2]),
@@ -1582,7 +1582,7 @@ void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x
       pairs_of(std::integral_constant<int, 32>{});
     }
   } else {
-    // one pixel per thread (arrays that are only 4-byte aligned, planes that are not whole 16-byte groups)
+    // one pixel per thread (planes that are not whole 16-byte groups)
     const uint32_t blocks = stream_grid(pg.total_groups, 1);
     if (C <= 4) {
       softmax_nd_reg_kernel<4, V, NLL, NT, 1, BWD><<<blocks, kBlock, 0, s>>>(pg, x, y, cat, nll, dy, dx);
@@ -1671,7 +1671,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
   for (uint64_t n0 = uint64_t(blockIdx.x) * SB; n0 < N; n0 += uint64_t(gridDim.x) * SB) {
     const uint32_t samples = (N - n0 < uint64_t(SB)) ? uint32_t(N - n0) : SB;
     const uint32_t n = samples * slab;
-    const uint32_t n4 = vec ? n / 4u : 0u;  // (the host checked that every tile starts on a 16-byte boundary)
+    const uint32_t n4 = vec ? n / 4u : 0u;  // (the host checked that every tile starts a whole number of 16-byte groups into the array)
     const float *xt = x + n0 * slab;
     float *yt = y + n0 * slab;
     // eight groups per thread are requested before the first is written to LDS (a slot past the tile's end reads
@@ -1767,7 +1767,7 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
                             float *nll, const float *dy, float *dx, bool ignore, hipStream_t s) {
   const uint32_t slab = P * C;
   // as many samples as fit, but no more than leaves every CU two workgroups; from four on a multiple of four,
-  // so that every tile starts on a 16-byte boundary
+  // so that every tile starts a whole number of 16-byte groups into the array
   uint32_t SB = kNdTileFloats / slab;
   const uint32_t spread = (N + 2u * uint32_t(device_cu_count()) - 1u) / (2u * uint32_t(device_cu_count()));
   if (SB > spread) SB = spread;
