@@ -526,7 +526,7 @@ __global__ __launch_bounds__(THREADS) void softmax_row_reglds_kernel(uint32_t K,
 // one row at a time leaves the memory system idle between the phases; two workgroups overlap them.)
 constexpr int kRowStreamThreads = 512;
 constexpr int kRowStreamHeld = 32 * kRowStreamThreads;  // values of a row that stay in LDS
-// MODE 0: 4-byte accesses.  MODE 1: 16-byte accesses, every row starts on a 16-byte boundary.  MODE 2: 16-byte
+// MODE 0: 4-byte accesses.  MODE 1: 16-byte accesses, every row is a whole number of 16-byte groups.  MODE 2: 16-byte
 // accesses to the aligned groups of the array from the start of the 128-byte line of y in which a row begins (x and
 // y, and dx, start equally far from a 16-byte boundary; `mis` is y's distance in floats from a line): every step of
 // a wave then covers whole lines of y, whatever the row length, and the values of a row's first and last groups
