@@ -73,8 +73,8 @@ MEASURED_TRAFFIC = {
     ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): (308434067, "bn_maps"),
     ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): (1610547205, "flat_maps"),
     ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): (637597563, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291270148, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671292527, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291264004, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671294575, "softmax"),
     ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): (192699228, "flat_maps"),
     ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): (192703324, "flat_maps"),
 }
@@ -89,10 +89,10 @@ TRAFFIC_FAMILY_SOURCES = {
     "softmax": ["common.hpp", "softmax.hip"],
 }
 TRAFFIC_FAMILY_FINGERPRINT = {
-    "bn_maps": "a3cf33780e6faed1",
-    "bn_reductions": "5049c23d0382fb4f",
-    "flat_maps": "33673a31b6d796e7",
-    "softmax": "0183ec9269a10ee9",
+    "bn_maps": "f1d2731d688bbd74",
+    "bn_reductions": "17e1672fd4657de8",
+    "flat_maps": "55a8a2fcc3e0ac85",
+    "softmax": "dda536fce5d8fc73",
 }
 
 
