@@ -1827,9 +1827,21 @@ ColTile nd_col_tile(uint32_t P, uint32_t C) {
     // Short planes: tiles of about the same width.  Planes that are not whole 32-byte pieces are left to the other
     // kernels unless a tile holds a whole plane: their runs start anywhere in a piece, and cut runs then share
     // pieces with their neighbours ([196, 128] 2.5 TB/s against 3.5).
-    if (P % 8u != 0) return ct;
+    // (from 256 pixels on they take the column tiles up to 128 classes, with ordinary stores, which the L2 merges:
+    // [676, 100] 3.1 -> 3.9 TB/s, [900, 65] 2.6 -> 4.0 against one pixel per thread; beyond 128 classes the kernels with
+    // eight lanes per pixel group are as fast or faster, [900, 150] 4.1 against 3.6)
+    if (P % 8u != 0 && (P < 256u || C > 128u)) return ct;
     const uint32_t tiles = (P + TP - 1) / TP;
-    TP = ((P + tiles - 1) / tiles + 3u) & ~3u;
+    const uint32_t width = (P + tiles - 1) / tiles;
+    if (P % 16u == 0) {
+      // runs of whole 64-byte pieces: a run that ends inside a piece shares it with the next tile's, and both
+      // write a part of it ([400, 128] in runs of 240 bytes 2.9 TB/s, [576, 200] in runs of 160 bytes 2.9)
+      TP = (width + 15u) & ~15u;
+      if (uint64_t(TP) * C > kColTileMaxFloats) TP -= 16u;
+      if (TP < 16u) return ct;
+    } else {
+      TP = (width + 3u) & ~3u;
+    }
   }
   ct.TP = TP;
   ct.L = 256u / TP;
@@ -1989,10 +2001,192 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
   const FastDiv div_tps(ct.tiles_per_sample), div_tp(ct.TP);
   const uint32_t xcd = P >= 1024 ? 1u : 0u;
   // logits in, probabilities (and the gradient) out: all streamed
-  const int nt = policy_for_outputs(stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal), y, dx);
+  // (streaming stores only where every run of a tile is whole 64-byte pieces, or a tile holds whole samples)
+  const int nt = (P % 16u == 0 || ct.TP >= P) ? policy_for_outputs(stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal), y, dx) : 0;
   with_stream_policy(nt, [&](auto policy) {
     softmax_nd_coltile_kernel<NLL, BWD, decltype(policy)::value><<<blocks, kBlock, lds_bytes, s>>>(
         P, C, ct.TP, ct.L, total_tiles, div_tps, div_tp, ignore ? 1u : 0u, xcd, x, y, cat, nll, dy, dx);
+  });
+}
+
+// Whole samples in registers, for short planes of whole 16-byte groups with many classes: one workgroup per sample,
+// whose G = P / 4 pixel groups times C classes lie contiguously in memory.  Thread t = phase * G + g holds pixel group
+// g of the classes phase, phase + PH, phase + 2 PH, ... (PH = threads / G phases, at most NS classes per thread), so
+// slot i of the workgroup's live threads is the contiguous run of G * PH groups that starts i * G * PH groups into
+// the sample: every access is 16 bytes per lane over whole runs of the array, whatever P is, x is read once, and
+// nothing but the PH partial maxima and sums of a pixel group goes through LDS.  A pixel's sum is the sum of its PH
+// partial sums in phase order, each added in class order: it depends on the shape and on nothing else.
+struct SampleReg {
+  uint32_t threads;  // 256, 512 or 1024: the kernel's launch bound
+  uint32_t ns;       // 8 or 16 slots per thread
+  uint32_t G, PH;
+  bool fits;
+};
+
+template <int NS, int THREADS, bool NLL, bool BWD, int NT>
+__global__ __launch_bounds__(THREADS) void softmax_nd_samplereg_kernel(uint32_t P, uint32_t C, uint32_t N, uint32_t G,
+                                                                      uint32_t PH, FastDiv div_g, uint32_t ignore,
+                                                                      const float *__restrict__ x,
+                                                                      float *__restrict__ y,
+                                                                      const uint32_t *__restrict__ cat,
+                                                                      float *__restrict__ nll,
+                                                                      const float *__restrict__ dy,
+                                                                      float *__restrict__ dx) {
+  static_assert(!BWD || NLL, "the backward pass needs the labels");
+  __shared__ f32x4 part_max[THREADS], part_sum[THREADS];
+  const uint32_t t = threadIdx.x;
+  const uint32_t live_threads = G * PH;
+  const bool live = t < live_threads;
+  uint32_t phase, g;
+  div_g.divmod(t, phase, g);
+  const size_t sample = size_t(P) * C;
+  const f32x4 ninf = PixVec<f32x4>::splat(kNegInf);
+  for (uint64_t n = blockIdx.x; n < N; n += gridDim.x) {
+    const f32x4 *xs = reinterpret_cast<const f32x4 *>(x + n * sample);
+    const size_t pix = n * P + 4u * g;
+    u32x4 lab = {0u, 0u, 0u, 0u};
+    f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (NLL && live) lab = load_stream<0>(reinterpret_cast<const u32x4 *>(cat + pix));
+    if (BWD && live) d = load_stream<0>(reinterpret_cast<const f32x4 *>(dy + pix));
+    f32x4 v[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const uint32_t c = uint32_t(i) * PH + phase;
+      v[i] = (live && c < C) ? load_stream<NT>(xs + (size_t(i) * live_threads + t)) : ninf;
+    }
+    f32x4 m = ninf;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) m = vmax(m, v[i]);
+    if (live) part_max[t] = m;
+    __syncthreads();
+    if (live) {
+      m = part_max[g];
+      for (uint32_t ph = 1; ph < PH; ++ph) m = vmax(m, part_max[ph * G + g]);
+    }
+    f32x4 sum = PixVec<f32x4>::splat(0.0f);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const uint32_t c = uint32_t(i) * PH + phase;
+      v[i] = (live && c < C) ? vexp(v[i] - m) : PixVec<f32x4>::splat(0.0f);
+      sum += v[i];
+    }
+    if (live) part_sum[t] = sum;
+    __syncthreads();
+    if (live) {
+      sum = part_sum[g];
+      for (uint32_t ph = 1; ph < PH; ++ph) sum += part_sum[ph * G + g];
+      const f32x4 inv = vrcp(sum);  // one correctly rounded reciprocal per pixel
+      if (BWD && ignore) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          if (lab[w] >= C) d[w] = 0.0f;
+        }
+      }
+      f32x4 *ys = reinterpret_cast<f32x4 *>(y + n * sample);
+      f32x4 *ds = BWD ? reinterpret_cast<f32x4 *>(dx + n * sample) : nullptr;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        const uint32_t c = uint32_t(i) * PH + phase;
+        if (c < C) {
+          const f32x4 pr = v[i] * inv;
+          store_stream<NT>(ys + (size_t(i) * live_threads + t), pr);
+          if (NLL) {
+            // -log of the stored probability, by the thread that holds the label's class
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              if (lab[w] == c) nll[pix + uint32_t(w)] = -logf(pr[w]);
+            }
+          }
+          if (BWD) {
+            f32x4 gr;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) gr[w] = d[w] * (pr[w] - float(lab[w] == c));
+            store_stream<NT>(ds + (size_t(i) * live_threads + t), gr);
+          }
+        }
+      }
+      if (NLL && phase == 0u) {  // a label out of range: NaN (0 with `ignore`)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          if (lab[w] >= C) nll[pix + uint32_t(w)] = ignore ? 0.0f : __builtin_nanf("");
+        }
+      }
+    }
+    // (part_max is written again only after the barrier above, part_sum only after the next one)
+  }
+}
+
+// Which form of the kernel a shape takes, if any.  Forms in the order they are tried: (threads, slots per thread)
+// with the workgroups of it that fit a CU by registers -- (256, 8) eight, (256, 16) and (512, 8) four, (512, 16) and
+// (1024, 8) two, (1024, 16) one.  The first form that holds the classes and keeps at least 64 KB of samples in
+// flight per CU is taken (a [36, 33] sample is 4.6 KB: eight of them leave the memory system idle, 3.1 TB/s against
+// 5.8 through the LDS tiles); at most 32 phases, since every thread reads all partial values of its pixel group
+// ([16, 200] with 64 phases: 4.2 TB/s against 5.8).  One workgroup of 1024 threads per CU loads, reduces and stores
+// in turn, 4.6-4.9 TB/s: taken only from 129 classes on, or for planes that are not whole 64-byte pieces, where the
+// other kernels run at 2.6-3.9.
+// Measured on 256 MB arrays, against the kernels that took these shapes before (LDS tiles, column tiles, one pixel
+// per thread, eight lanes per pixel group): [196, 64] 4.7 -> 5.5 TB/s, [196, 100] 3.1 -> 5.3, [196, 150] 3.9 -> 5.1,
+// [196, 200 / 256 / 300] 3.1 / 3.3 / 2.7 -> 4.6, [100, 100 ... 300] 2.6-4.0 -> 5.3-5.8, [36, 256] 2.1 -> 5.7,
+// [256, 150] 3.0 -> 4.7, [400, 150] 2.6 -> 4.9, [64, 33] 4.8 -> 6.1, [400, 33] 4.6 -> 5.9; within 6 % either way at
+// [64, 100], [100, 33], [196, 33], [36, 200].
+SampleReg nd_sample_reg(uint32_t P, uint32_t C) {
+  SampleReg sr = {0, 0, 0, 0, false};
+  if (tuning().nd_sample_reg == 0) return sr;
+  if (P % 4u != 0 || P < 8u || P >= 1024u || C <= 32u) return sr;  // (longer planes never hold 33 classes in a form that is taken)
+  // (samples of up to 32 KB on planes of 96 pixels and more keep the LDS tile, where enough threads of a tile have a
+  // pixel to walk: [196, 33] 5.9 TB/s against 5.5, [100, 48] 5.7 against 5.5)
+  if (C <= 64u && P >= 96u && uint64_t(P) * C <= kNdTileMaxSample && nd_tile_fits(P, C)) return sr;
+  const uint32_t G = P / 4u;
+  const uint64_t sample_bytes = uint64_t(P) * C * sizeof(float);
+  const uint32_t forms[6][3] = {{256, 8, 8}, {256, 16, 4}, {512, 8, 4}, {512, 16, 2}, {1024, 8, 2}, {1024, 16, 1}};
+  for (const auto &f : forms) {
+    uint32_t PH = f[0] / G;
+    if (PH > 32u) PH = 32u;
+    if (PH == 0 || uint64_t(PH) * f[1] < C) continue;
+    if (f[2] * sample_bytes < (64u << 10)) return sr;  // (the later forms keep no more in flight)
+    if (f[2] == 1u && C <= 128u && P % 16u == 0) return sr;  // (planes of whole 64-byte pieces: the column tiles, 5.0-5.8 TB/s)
+    sr.threads = f[0];
+    sr.ns = f[1];
+    sr.G = G;
+    sr.PH = PH;
+    sr.fits = true;
+    return sr;
+  }
+  return sr;
+}
+
+template <bool NLL, bool BWD>
+void launch_softmax_nd_samplereg(const SampleReg &sr, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
+                                 const uint32_t *cat, float *nll, const float *dy, float *dx, bool ignore,
+                                 hipStream_t s) {
+  const uint32_t max_blocks = 1u << 24;
+  const uint32_t blocks = N < max_blocks ? N : max_blocks;
+  const uint32_t live_threads = sr.G * sr.PH;
+  const uint32_t launch_threads = (live_threads + kWave - 1u) / kWave * kWave;
+  const FastDiv div_g(sr.G);
+  // streaming stores only where every step of every sample starts on a 64-byte boundary
+  const bool whole_pieces = (uint64_t(P) * C) % 16u == 0 && live_threads % 4u == 0;
+  const int nt = whole_pieces ? policy_for_outputs(stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal), y, dx) : 0;
+  with_stream_policy(nt, [&](auto policy) {
+    constexpr int NT = decltype(policy)::value;
+    auto go = [&](auto ns, auto threads) {
+      softmax_nd_samplereg_kernel<decltype(ns)::value, decltype(threads)::value, NLL, BWD, NT>
+          <<<blocks, launch_threads, 0, s>>>(P, C, N, sr.G, sr.PH, div_g, ignore ? 1u : 0u, x, y, cat, nll, dy, dx);
+    };
+    auto with_ns = [&](auto threads) {
+      if (sr.ns == 8) {
+        go(std::integral_constant<int, 8>{}, threads);
+      } else {
+        go(std::integral_constant<int, 16>{}, threads);
+      }
+    };
+    if (sr.threads == 256) {
+      with_ns(std::integral_constant<int, 256>{});
+    } else if (sr.threads == 512) {
+      with_ns(std::integral_constant<int, 512>{});
+    } else {
+      with_ns(std::integral_constant<int, 1024>{});
+    }
   });
 }
 
@@ -2018,7 +2212,10 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
   hipStream_t s = as_stream(stream);
   const bool vec = nd_vec(P);
   const ColTile ct = nd_col_tile(P, C);
-  if (nd_tile_fits(P, C)) {
+  const SampleReg sr = nd_sample_reg(P, C);
+  if (sr.fits) {
+    launch_softmax_nd_samplereg<false, false>(sr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+  } else if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (vec && ct.fits) {
     launch_softmax_nd_coltile<false, false>(ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
@@ -2252,6 +2449,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
+  } else if (const SampleReg sr = nd_sample_reg(prefix_dim, dim0); sr.fits) {
+    launch_softmax_nd_samplereg<true, false>(sr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
+                                             false, as_stream(stream));
+    note_launch(__func__);
   } else if (nd_tile_fits(prefix_dim, dim0)) {
     launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                         as_stream(stream));
@@ -2290,6 +2491,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   if (len == 0) return;
   if (prefix_dim == 1) {  // the class axis is contiguous: the row form
     launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
+  } else if (const SampleReg sr = nd_sample_reg(prefix_dim, dim0); sr.fits) {
+    launch_softmax_nd_samplereg<true, true>(sr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
+                                            as_stream(stream));
+    note_launch(__func__);
   } else if (nd_tile_fits(prefix_dim, dim0)) {
     launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                        as_stream(stream));

@@ -198,7 +198,11 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
                                    # tiles of all classes of a run of pixels in LDS
                                    (64, 300, 3), (196, 150, 2), (1028, 200, 1), (20, 70, 5), (16, 944, 1), (1056, 256, 2),
                                    # samples of up to 63 KB with a tile to themselves
-                                   (196, 70, 3), (196, 82, 2), (100, 100, 2), (36, 128, 3)])
+                                   (196, 70, 3), (196, 82, 2), (100, 100, 2), (36, 128, 3),
+                                   # whole samples in registers: the forms of the kernel
+                                   (100, 33, 3), (36, 256, 3), (400, 40, 2), (784, 40, 2), (196, 200, 2), (196, 320, 1),
+                                   # column tiles over planes that are not whole 32-byte pieces
+                                   (676, 100, 1), (900, 65, 2)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

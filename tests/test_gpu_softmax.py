@@ -255,6 +255,14 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # samples of up to 63 KB with a tile to themselves (more than 32 classes, planes that are not whole 64-byte
              # pieces), the largest that fits and one class more, and a short plane that the column tiles keep
              (196, 70, 3), (196, 82, 2), (196, 83, 2), (100, 100, 3), (36, 128, 3), (900, 17, 2), (252, 64, 2),
+             # whole samples in registers (short planes of whole 16-byte groups, more than 32 classes): every form of
+             # the kernel -- 256, 512 and 1024 threads with 8 and 16 slots each --, the most classes the largest
+             # form holds at 49 pixel groups (320) and one more, which goes back to the other kernels
+             (64, 33, 5), (100, 33, 3), (36, 256, 3), (400, 40, 2), (784, 40, 2), (196, 200, 2), (196, 300, 2),
+             (196, 320, 1), (196, 321, 1),
+             # column tiles over planes that are not whole 32-byte pieces (256 pixels and more, 65 to 128 classes,
+             # too many pixel groups for a sample in registers), and one class more
+             (676, 100, 1), (900, 65, 2), (1012, 128, 1), (900, 129, 1),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
@@ -295,7 +303,7 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
 
 
 @pytest.mark.parametrize("P,C,N", [(64, 19, 3), (196, 19, 5), (196, 70, 3), (64, 300, 2), (1056, 200, 1), (2048, 19, 2),
-                                   (1028, 300, 1), (36, 128, 3)])
+                                   (1028, 300, 1), (36, 128, 3), (196, 150, 2), (400, 40, 2), (784, 40, 1), (196, 200, 2), (900, 65, 1)])
 def test_softmax_nd_arrays_that_lie_differently(oracle, P, C, N):
     # every n-d kernel family with arrays at different element offsets from a 16-byte boundary: the 16-byte forms
     # need all of a launch's arrays aligned, and any mix must still give the 4-byte forms' (correct) results;
@@ -374,13 +382,14 @@ def test_softmax_nd_tile_of_fewer_than_four_floats(oracle, P, C, N, off):
     assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "fused dx vs fp32 of its own p")
 
 
-@pytest.mark.parametrize("P", [8, 1028])
+@pytest.mark.parametrize("P", [8, 36, 100, 1028])
 @pytest.mark.parametrize("C", [3, 19, 40, 100, 200, 300])
 def test_softmax_nd_special_values(oracle, C, P):
     # register-resident (2 or 8 lanes per pixel group up to 256 classes; one pixel per thread without 16-byte
     # accesses up to 128) and streaming kernels: -inf entries get probability 0, a NaN
     # poisons its pixel only, a pixel of +-1e30 and one of large equal values do not overflow, widely spread logits
-    # keep their small probabilities to the relative bar.  P = 8 goes through the LDS tile up to 64 classes.
+    # keep their small probabilities to the relative bar.  P = 8 goes through the LDS tile up to 64 classes; P = 36
+    # and 100 keep whole samples in registers from 100 and 40 classes on.
     N = 2
     g = np.random.default_rng(C)
     x = g.standard_normal((N, C, P)).astype(F32)

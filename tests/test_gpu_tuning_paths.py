@@ -30,6 +30,10 @@ PROFILES = {
     "long_rows_streamed": {15: 0},
     "long_rows_streamed_nontemporal": {15: 0, 5: 0},
     "long_rows_half_in_lds_nontemporal": {5: 0},
+    # knob 17: n-d softmax over short planes with more than 32 classes keeps whole samples in registers; 0 sends
+    # them to the LDS tiles, the column tiles and the register kernels that split a pixel group over lanes
+    "nd_short_planes_through_tiles": {17: 0},
+    "nd_short_planes_through_tiles_nontemporal": {17: 0, 5: 0},
 }
 
 
@@ -64,7 +68,8 @@ def test_softmax_under_tuning(tuned, oracle):
         for name in T_sm.ROW_ENTRY_POINTS:
             T_sm.test_softmax_rows(oracle, name, K, R)
     T_sm.test_softmax_cat_nll_and_bwd_rows(oracle, 1000, 256)
-    for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3), (16, 200, 2), (1024, 256, 2)]:
+    for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3), (16, 200, 2), (1024, 256, 2),
+                    (196, 70, 3), (100, 100, 3), (196, 150, 2), (64, 300, 3), (196, 200, 2), (256, 65, 2), (324, 70, 2)]:
         T_sm.test_softmax_nd_all_symbols(oracle, P, C, N)
 
 
@@ -76,3 +81,5 @@ def test_additive_under_tuning(tuned, oracle):
     for masked in (False, True):
         T_add.test_fused_batch_norm_equals_the_launch_sequence(oracle, 784, 16, 32, masked)
     T_add.test_fused_softmax_nd_nll_equals_the_two_launches(oracle, 2048, 19, 2)
+    for P, C, N in [(196, 82, 2), (64, 300, 3), (196, 200, 2)]:
+        T_add.test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N)
