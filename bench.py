@@ -73,8 +73,8 @@ MEASURED_TRAFFIC = {
     ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): (308434067, "bn_maps"),
     ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): (1610547205, "flat_maps"),
     ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): (637597563, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291264004, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671294575, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291356156, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671292527, "softmax"),
     ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): (192699228, "flat_maps"),
     ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): (192703324, "flat_maps"),
 }
@@ -89,10 +89,10 @@ TRAFFIC_FAMILY_SOURCES = {
     "softmax": ["common.hpp", "softmax.hip"],
 }
 TRAFFIC_FAMILY_FINGERPRINT = {
-    "bn_maps": "f1d2731d688bbd74",
-    "bn_reductions": "17e1672fd4657de8",
-    "flat_maps": "55a8a2fcc3e0ac85",
-    "softmax": "dda536fce5d8fc73",
+    "bn_maps": "4d02d8d7280b081e",
+    "bn_reductions": "10f7ba7330302d99",
+    "flat_maps": "c6691b9dd66bc786",
+    "softmax": "09817018d533cf9e",
 }
 
 
@@ -479,7 +479,7 @@ def shape_sweep(torch, gpu):
             "K": K, "R": R,
             "softmax_packed_block": rate(lambda i: gpu.call("anode_gpu_softmax_packed_block_f32", K, R, x[i % 3],
                                                             x[3 + i % 3]), 8 * n)})
-    for P in (65536, 196):
+    for P in (65536, 400, 196):
         for C in (2, 4, 19, 32, 33, 64, 100, 128, 150, 256, 300):
             N = min(total // (P * C), 1 << 20)
             if N < 1:
