@@ -201,6 +201,13 @@ for i in range(20 * SCALE):
     C = log_uniform(_g, 1, 700)
     ND_CASES.append((max(1, min(log_uniform(_g, 1, 40000), (BUDGET >> 1) // C)), C, log_uniform(_g, 1, 4),
                      int(_g.integers(0, 4))))
+# short planes of whole 16-byte groups with more than 32 classes: the kernels that keep whole samples in registers
+# or cut planes into column tiles, which a uniformly drawn P seldom reaches
+for i in range(12 * SCALE):
+    _g = np.random.default_rng(550000 + i)
+    C = log_uniform(_g, 33, 700)
+    ND_CASES.append((min(4 * log_uniform(_g, 2, 255), max(4, ((BUDGET >> 1) // C) & ~3)), C, log_uniform(_g, 1, 6),
+                     int(_g.integers(0, 4))))
 
 
 @pytest.mark.parametrize("P,C,N,offset", ND_CASES)
