@@ -276,6 +276,7 @@ struct Tuning {
   Knob nd_bwd_flat_max_plane;    // n-d NLL backward: planes of up to this many pixels are walked as a flat array
   Knob nd_pair_ballast;          // KiB of unused LDS per workgroup of the two-lane n-d softmax forward kernel at 17 to 24 classes (caps the workgroups per CU; 0: no cap)
   Knob nd_sample_reg;            // n-d softmax, short planes with more than 32 classes: whole samples in registers (1) or the tile kernels (0)
+  Knob nd_colreg;                // n-d softmax, 33 to 512 classes on planes of 128 pixels and more: column tiles in registers (1) or the other kernels (0)
   Knob row_reglds;               // row softmax, rows of whole 16-byte groups held half in LDS, half in registers: 1 for 16385 to 32768 classes, 2 for 32769 to 65536
 };
 

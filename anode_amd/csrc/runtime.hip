@@ -52,6 +52,7 @@ Tuning g_tuning = {
     /*nd_bwd_flat_max_plane=*/{{131072}},
     /*nd_pair_ballast=*/{{32}},
     /*nd_sample_reg=*/{{1}},
+    /*nd_colreg=*/{{1}},
     /*row_reglds=*/{{3}},
     };
 
@@ -430,7 +431,8 @@ ANODE_EXPORT uint32_t anode_gpu_fastdiv_probe(uint32_t n, uint32_t d) { return a
 // 3 nontemporal (0, 1 or 3: streaming loads without streaming stores is not a policy the maps are built for),
 // 4 reduce_nontemporal, 5 nt_min_bytes, 6 reduce_min_tile, 7 nt_store_min_bytes, 8 reduce_tile_pos,
 // 9 reduce_lanes, 10 reduce_single_pass_grid, 11 reduce_lanes_max_ctiles, 12 reduce_lanes_min_run, 13 nd_xcd_mask,
-// 14 nd_bwd_flat_max_plane, 15 row_reglds, 16 nd_pair_ballast, 17 nd_sample_reg.  Returns the previous value; a
+// 14 nd_bwd_flat_max_plane, 15 row_reglds, 16 nd_pair_ballast, 17 nd_sample_reg,
+// 18 nd_colreg.  Returns the previous value; a
 // negative value only reads.  Returns -1, and changes nothing, for an unknown knob or a value the knob does not take.
 ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
   anode::Tuning &t = anode::tuning();
@@ -453,6 +455,7 @@ ANODE_EXPORT int anode_gpu_set_tuning(int knob, int value) {
     case 15: slot = &t.row_reglds; break;
     case 16: slot = &t.nd_pair_ballast; break;
     case 17: slot = &t.nd_sample_reg; break;
+    case 18: slot = &t.nd_colreg; break;
     default: return -1;
   }
   if (knob == 3 && value >= 0 && value != 0 && value != 1 && value != 3) return -1;

@@ -2016,6 +2016,12 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
 // the sample: every access is 16 bytes per lane over whole runs of the array, whatever P is, x is read once, and
 // nothing but the PH partial maxima and sums of a pixel group goes through LDS.  A pixel's sum is the sum of its PH
 // partial sums in phase order, each added in class order: it depends on the shape and on nothing else.
+struct ColReg {  // the tiling of softmax_nd_colreg_kernel, further down
+  uint32_t ns, Gt, PH, tiles, xcd;
+  bool fits;
+};
+ColReg nd_col_reg(uint32_t P, uint32_t C);
+
 struct SampleReg {
   uint32_t threads;  // 256, 512 or 1024: the kernel's launch bound
   uint32_t ns;       // 8 or 16 slots per thread
@@ -2144,6 +2150,9 @@ SampleReg nd_sample_reg(uint32_t P, uint32_t C) {
     if (PH > 32u) PH = 32u;
     if (PH == 0 || uint64_t(PH) * f[1] < C) continue;
     if (f[2] * sample_bytes < (64u << 10)) return sr;  // (the later forms keep no more in flight)
+    // (from 128 pixels on, tiles of the planes in registers are faster than a sample per 1024 threads: [256, 150] 4.8
+    // against 5.9 TB/s, [196, 200] 4.4 against 5.2)
+    if (f[0] == 1024u && nd_col_reg(P, C).fits) return sr;
     if (f[2] == 1u && C <= 128u && P % 16u == 0) return sr;  // (planes of whole 64-byte pieces: the column tiles, 5.0-5.8 TB/s)
     sr.threads = f[0];
     sr.ns = f[1];
@@ -2159,7 +2168,8 @@ template <bool NLL, bool BWD>
 void launch_softmax_nd_samplereg(const SampleReg &sr, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                                  const uint32_t *cat, float *nll, const float *dy, float *dx, bool ignore,
                                  hipStream_t s) {
-  const uint32_t max_blocks = 1u << 24;
+  uint32_t max_blocks = 1u << 24;
+  if (tuning().flat_wg_per_cu > 0) max_blocks = uint32_t(device_cu_count()) * uint32_t(tuning().flat_wg_per_cu);  // (the tests' way into the loop over samples)
   const uint32_t blocks = N < max_blocks ? N : max_blocks;
   const uint32_t live_threads = sr.G * sr.PH;
   const uint32_t launch_threads = (live_threads + kWave - 1u) / kWave * kWave;
@@ -2186,6 +2196,185 @@ void launch_softmax_nd_samplereg(const SampleReg &sr, uint32_t P, uint32_t C, ui
       with_ns(std::integral_constant<int, 512>{});
     } else {
       with_ns(std::integral_constant<int, 1024>{});
+    }
+  });
+}
+
+// Column tiles in registers, for 33 to 512 classes on planes of 128 pixels and more in whole 16-byte groups: the
+// kernel above with a workgroup per run of Gt pixel groups of one sample instead of per sample.  Thread t =
+// phase * Gt + g holds pixel group g of the tile for the classes phase, phase + PH, ...: a wave reads, per slot, 64 / Gt
+// runs of Gt * 16 bytes, one per plane, and x is read once with nothing but the partial maxima and sums in LDS (the
+// LDS column tiles below move every value through LDS five times).  Against the kernels that took these shapes before
+// (eight lanes per pixel group up to 256 classes, LDS column tiles, the two-pass kernel beyond), 256 MB arrays:
+// [65536, 64] 5.3 -> 5.9 TB/s, [65536, 200] 4.9 -> 5.5, [65536, 256] 4.3 -> 5.4, [65536, 300] 4.3 -> 5.1,
+// [65536, 512] 3.5 -> 4.9, [2048, 256] 4.7 -> 5.9, [784, 300] 3.7 -> 5.1, [256, 300] 3.5 -> 5.6; planes that are not
+// whole 128-byte lines, with neighbouring tiles on one XCD so that the lines they share are fetched once:
+// [900, 100] 3.9 -> 5.6, [900, 200] 3.1 -> 5.3, [1028, 64] 4.0 -> 5.6, [676, 128] 3.8 -> 5.5.
+template <int NS, int THREADS, bool NLL, bool BWD, int NT>
+__global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4, uint32_t C, uint32_t Gt, uint32_t PH,
+                                                                   uint32_t total_tiles, FastDiv div_gt,
+                                                                   FastDiv div_tiles, uint32_t ignore, uint32_t xcd,
+                                                                   const float *__restrict__ x, float *__restrict__ y,
+                                                                   const uint32_t *__restrict__ cat,
+                                                                   float *__restrict__ nll,
+                                                                   const float *__restrict__ dy,
+                                                                   float *__restrict__ dx) {
+  static_assert(!BWD || NLL, "the backward pass needs the labels");
+  __shared__ f32x4 part_max[THREADS], part_sum[THREADS];
+  const uint32_t t = threadIdx.x;
+  uint32_t phase, g;
+  div_gt.divmod(t, phase, g);
+  const f32x4 ninf = PixVec<f32x4>::splat(kNegInf);
+  for (uint32_t b0 = blockIdx.x; b0 < total_tiles; b0 += gridDim.x) {
+    const uint32_t b = (xcd && gridDim.x == total_tiles) ? xcd_contiguous(b0, total_tiles) : b0;
+    uint32_t n, ti;
+    div_tiles.divmod(b, n, ti);
+    const uint32_t g0 = ti * Gt;
+    const uint32_t gt = P4 - g0 < Gt ? P4 - g0 : Gt;
+    const bool live = phase < PH && g < gt;
+    const size_t first = size_t(n) * C * P4 + g0 + g;  // in 16-byte groups: class c of this thread's pixels is c * P4 further
+    const f32x4 *xs = reinterpret_cast<const f32x4 *>(x) + first;
+    const size_t pix = (size_t(n) * P4 + g0 + g) * 4u;
+    u32x4 lab = {0u, 0u, 0u, 0u};
+    f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (NLL && live) lab = load_stream<0>(reinterpret_cast<const u32x4 *>(cat + pix));
+    if (BWD && live) d = load_stream<0>(reinterpret_cast<const f32x4 *>(dy + pix));
+    f32x4 v[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const uint32_t c = uint32_t(i) * PH + phase;
+      v[i] = (live && c < C) ? load_stream<NT>(xs + size_t(c) * P4) : ninf;
+    }
+    f32x4 m = ninf;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) m = vmax(m, v[i]);
+    if (live) part_max[t] = m;
+    __syncthreads();
+    if (live) {
+      m = part_max[g];
+      for (uint32_t ph = 1; ph < PH; ++ph) m = vmax(m, part_max[ph * Gt + g]);
+    }
+    f32x4 sum = PixVec<f32x4>::splat(0.0f);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const uint32_t c = uint32_t(i) * PH + phase;
+      v[i] = (live && c < C) ? vexp(v[i] - m) : PixVec<f32x4>::splat(0.0f);
+      sum += v[i];
+    }
+    if (live) part_sum[t] = sum;
+    __syncthreads();
+    if (live) {
+      sum = part_sum[g];
+      for (uint32_t ph = 1; ph < PH; ++ph) sum += part_sum[ph * Gt + g];
+      const f32x4 inv = vrcp(sum);
+      if (BWD && ignore) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          if (lab[w] >= C) d[w] = 0.0f;
+        }
+      }
+      f32x4 *ys = reinterpret_cast<f32x4 *>(y) + first;
+      f32x4 *ds = BWD ? reinterpret_cast<f32x4 *>(dx) + first : nullptr;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        const uint32_t c = uint32_t(i) * PH + phase;
+        if (c < C) {
+          const f32x4 pr = v[i] * inv;
+          store_stream<NT>(ys + size_t(c) * P4, pr);
+          if (NLL) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              if (lab[w] == c) nll[pix + uint32_t(w)] = -logf(pr[w]);
+            }
+          }
+          if (BWD) {
+            f32x4 gr;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) gr[w] = d[w] * (pr[w] - float(lab[w] == c));
+            store_stream<NT>(ds + size_t(c) * P4, gr);
+          }
+        }
+      }
+      if (NLL && phase == 0u) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          if (lab[w] >= C) nll[pix + uint32_t(w)] = ignore ? 0.0f : __builtin_nanf("");
+        }
+      }
+    }
+  }
+}
+
+// The tile a shape takes.  512 threads; 8 slots per thread up to 128 classes (256 on planes that are not whole
+// 128-byte lines), 16 beyond; runs of as many pixel groups as the threads then hold, up to 32 (64 up to 64 classes, 24
+// on planes that are not whole lines: [900, 100] 5.6 TB/s in runs of 24 groups, 5.4 in runs of 32), a multiple of 8
+// groups on planes of whole lines and of 4 otherwise, evened out over the tiles of a plane without adding a tile.
+// (Shorter runs that divide the plane exactly were slower where they fell under 16 groups: [324, 100] in runs of 12
+// 3.7 TB/s, of 24 5.5.)
+// Measured alternatives: 256 and 1024 threads are within a few per cent either way at most shapes and 10 % behind at
+// some; dealing the tiles per XCD costs 3-7 % on planes of whole lines.
+ColReg nd_col_reg(uint32_t P, uint32_t C) {
+  ColReg cr = {0, 0, 0, 0, 0, false};
+  if (tuning().nd_colreg == 0) return cr;
+  if (P % 4u != 0 || P < 128u || C <= 32u || C > 512u) return cr;
+  const uint32_t P4 = P / 4u;
+  const bool lines = P4 % 8u == 0;
+  const uint32_t ns = (C <= 128u || (!lines && C <= 256u)) ? 8u : 16u;
+  const uint32_t ph_need = (C + ns - 1u) / ns;  // at most 32
+  const uint32_t step = lines ? 8u : 4u;
+  uint32_t gt_max = 512u / ph_need;
+  const uint32_t cap = C <= 64u ? 64u : (lines ? 32u : 24u);
+  if (gt_max > cap) gt_max = cap;
+  gt_max &= ~(step - 1u);
+  if (gt_max < step) gt_max = step;  // (512 / 32 = 16 groups at the least: never below a step)
+  // Planes of up to 1024 pixels where the plane and the sample are powers of two: runs one step shorter, which do not
+  // divide the plane, so that the tiles of a plane are not all alike: [1024, 64] 5.0 TB/s in four runs of 64 groups per
+  // 4 KB plane, 6.2 in runs of 56; [1024, 256] 5.4 -> 5.7 and [512, 256] 5.2 -> 5.6 in runs of 24 instead of 32,
+  // [1024, 128] 5.8 -> 6.0.  (Longer planes prefer the even division: [2048, 256] 5.9 in runs of 32, 5.6 in runs of 24;
+  // so do other class counts: [1024, 33 / 48 / 56] 6.2-6.3 in runs of 64, 5.7-5.8 in runs of 56.)
+  const bool pow2_sample = P4 <= 256u && (P & (P - 1u)) == 0 && (C & (C - 1u)) == 0;
+  if (pow2_sample && gt_max >= 3u * step && P4 > gt_max) gt_max -= step;  // (not below 16 groups)
+  uint32_t Gt = P4;
+  if (P4 > gt_max) {
+    // as many tiles per plane as runs of gt_max groups make, evened out ([196, 300]: 49 groups as 20 + 20 + 9 instead
+    // of 24 + 24 + 1)
+    const uint32_t per_plane = (P4 + gt_max - 1u) / gt_max;
+    Gt = ((P4 + per_plane - 1u) / per_plane + step - 1u) & ~(step - 1u);
+  }
+  uint32_t PH = 512u / Gt;
+  if (PH > 32u) PH = 32u;
+  if (uint64_t(PH) * ns < C) return cr;
+  cr.ns = ns;
+  cr.Gt = Gt;
+  cr.PH = PH;
+  cr.tiles = (P4 + Gt - 1u) / Gt;
+  cr.xcd = lines ? 0u : 1u;
+  cr.fits = true;
+  return cr;
+}
+
+template <bool NLL, bool BWD>
+void launch_softmax_nd_colreg(const ColReg &cr, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
+                              const uint32_t *cat, float *nll, const float *dy, float *dx, bool ignore,
+                              hipStream_t s) {
+  const uint32_t P4 = P / 4u;
+  const uint64_t total = uint64_t(cr.tiles) * N;  // at most len / 128: a tile is 33 classes of 4 pixel groups or more
+  uint32_t max_blocks = 1u << 24;
+  if (tuning().flat_wg_per_cu > 0) max_blocks = uint32_t(device_cu_count()) * uint32_t(tuning().flat_wg_per_cu);  // (the tests' way into the loop over tiles)
+  const uint32_t blocks = total < max_blocks ? uint32_t(total) : max_blocks;
+  const uint32_t launch_threads = (cr.Gt * cr.PH + kWave - 1u) / kWave * kWave;
+  const FastDiv div_gt(cr.Gt), div_tiles(cr.tiles);
+  // streaming stores only where every run of a tile is whole 64-byte pieces
+  const bool whole_pieces = P % 16u == 0 && cr.Gt % 4u == 0;
+  const int nt = whole_pieces ? policy_for_outputs(stream_policy(size_t(P) * C * N * sizeof(float), tuning().nontemporal), y, dx) : 0;
+  with_stream_policy(nt, [&](auto policy) {
+    constexpr int NT = decltype(policy)::value;
+    if (cr.ns == 8) {
+      softmax_nd_colreg_kernel<8, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
+          P4, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
+    } else {
+      softmax_nd_colreg_kernel<16, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
+          P4, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
     }
   });
 }
@@ -2217,6 +2406,8 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     launch_softmax_nd_samplereg<false, false>(sr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+  } else if (const ColReg cr = nd_col_reg(P, C); cr.fits) {
+    launch_softmax_nd_colreg<false, false>(cr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (vec && ct.fits) {
     launch_softmax_nd_coltile<false, false>(ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (nd_one_pixel_per_thread(P, C, vec)) {
@@ -2457,6 +2648,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                         as_stream(stream));
     note_launch(__func__);
+  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits) {
+    launch_softmax_nd_colreg<true, false>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
+                                          as_stream(stream));
+    note_launch(__func__);
   } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0); ct.fits) {
     launch_softmax_nd_coltile<true, false>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
                                            false, as_stream(stream));
@@ -2498,6 +2693,10 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   } else if (nd_tile_fits(prefix_dim, dim0)) {
     launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                        as_stream(stream));
+    note_launch(__func__);
+  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits) {
+    launch_softmax_nd_colreg<true, true>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
+                                         as_stream(stream));
     note_launch(__func__);
   } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0);
              ct.fits) {

@@ -440,13 +440,13 @@ import json, sys
 sys.path.insert(0, %r)
 from anode_amd import _lib
 lib = _lib.load()
-print(json.dumps([lib.cdll.anode_gpu_set_tuning(k, -1) for k in range(19)]))
+print(json.dumps([lib.cdll.anode_gpu_set_tuning(k, -1) for k in range(20)]))
 """ % (_lib.REPO_ROOT,)
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120, check=True)
     import json
     v = json.loads(r.stdout)
     assert v[0] == 0                      # flat maps: one 16-byte group per thread on a full grid
-    assert v[1] == -1 and v[18] == -1     # no such knobs
+    assert v[1] == -1 and v[19] == -1     # no such knobs
     assert v[3] == 3 and v[4] == 2        # streaming loads and stores in the maps, streaming loads in the reductions
     assert v[5] == 192 << 20 and v[7] == 16 << 20
     assert v[9] == 1 and v[10] == 256 and v[11] == 2048 and v[12] == 128
@@ -455,6 +455,7 @@ print(json.dumps([lib.cdll.anode_gpu_set_tuning(k, -1) for k in range(19)]))
     assert v[15] == 3                     # rows of 16385 to 65536 classes: half in LDS, half in registers
     assert v[16] == 32                    # n-d softmax forward at 17 to 24 classes: five workgroups per CU
     assert v[17] == 1                     # n-d softmax, short planes of many classes: whole samples in registers
+    assert v[18] == 1                     # n-d softmax, 33 to 512 classes on longer planes: column tiles in registers
 
 
 def test_product_package_never_reaches_the_oracle():

@@ -202,7 +202,9 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
                                    # whole samples in registers: the forms of the kernel
                                    (100, 33, 3), (36, 256, 3), (400, 40, 2), (784, 40, 2), (196, 200, 2), (196, 320, 1),
                                    # column tiles over planes that are not whole 32-byte pieces
-                                   (676, 100, 1), (900, 65, 2)])
+                                   (676, 100, 1), (900, 65, 2),
+                                   # column tiles in registers
+                                   (128, 33, 3), (132, 512, 2), (900, 300, 1), (400, 200, 2), (2048, 257, 1), (4096, 64, 1)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

@@ -263,6 +263,11 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # column tiles over planes that are not whole 32-byte pieces (256 pixels and more, 65 to 128 classes,
              # too many pixel groups for a sample in registers), and one class more
              (676, 100, 1), (900, 65, 2), (1012, 128, 1), (900, 129, 1),
+             # column tiles in registers (33 to 512 classes, planes of 128 pixels and more in whole 16-byte groups):
+             # the fewest and the most classes and one more, the shortest plane and the next shorter one, 8 and 16
+             # slots per thread, ragged last tiles, planes that are and are not whole 128-byte lines
+             (128, 33, 3), (124, 300, 2), (132, 512, 2), (1028, 513, 1), (900, 300, 1), (400, 200, 2), (4100, 40, 1),
+             (2048, 257, 1), (1024, 512, 1), (324, 256, 2), (4096, 64, 1),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
@@ -303,7 +308,8 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
 
 
 @pytest.mark.parametrize("P,C,N", [(64, 19, 3), (196, 19, 5), (196, 70, 3), (64, 300, 2), (1056, 200, 1), (2048, 19, 2),
-                                   (1028, 300, 1), (36, 128, 3), (196, 150, 2), (400, 40, 2), (784, 40, 1), (196, 200, 2), (900, 65, 1)])
+                                   (1028, 300, 1), (36, 128, 3), (196, 150, 2), (400, 40, 2), (784, 40, 1), (196, 200, 2), (900, 65, 1), (900, 300, 1),
+                                   (2048, 257, 1)])
 def test_softmax_nd_arrays_that_lie_differently(oracle, P, C, N):
     # every n-d kernel family with arrays at different element offsets from a 16-byte boundary: the 16-byte forms
     # need all of a launch's arrays aligned, and any mix must still give the 4-byte forms' (correct) results;
@@ -382,14 +388,15 @@ def test_softmax_nd_tile_of_fewer_than_four_floats(oracle, P, C, N, off):
     assert_bit_exact(host(dx), oracle.softmax_nd_cat_nll_bwd(P, C, N, dy, p, lab), "fused dx vs fp32 of its own p")
 
 
-@pytest.mark.parametrize("P", [8, 36, 100, 1028])
+@pytest.mark.parametrize("P", [8, 36, 100, 1028, 2048])
 @pytest.mark.parametrize("C", [3, 19, 40, 100, 200, 300])
 def test_softmax_nd_special_values(oracle, C, P):
     # register-resident (2 or 8 lanes per pixel group up to 256 classes; one pixel per thread without 16-byte
     # accesses up to 128) and streaming kernels: -inf entries get probability 0, a NaN
     # poisons its pixel only, a pixel of +-1e30 and one of large equal values do not overflow, widely spread logits
     # keep their small probabilities to the relative bar.  P = 8 goes through the LDS tile up to 64 classes; P = 36
-    # and 100 keep whole samples in registers from 100 and 40 classes on.
+    # and 100 keep whole samples in registers from 100 and 40 classes on; P = 1028 and 2048 take column tiles in
+    # registers from 40 classes on (planes that are not, and are, whole 128-byte lines).
     N = 2
     g = np.random.default_rng(C)
     x = g.standard_normal((N, C, P)).astype(F32)

@@ -34,6 +34,10 @@ PROFILES = {
     # them to the LDS tiles, the column tiles and the register kernels that split a pixel group over lanes
     "nd_short_planes_through_tiles": {17: 0},
     "nd_short_planes_through_tiles_nontemporal": {17: 0, 5: 0},
+    # knob 18: n-d softmax with 33 to 512 classes on planes of 128 pixels and more takes column tiles in registers; 0
+    # sends them to the kernels with eight lanes per pixel group, the LDS column tiles and the two-pass kernel
+    "nd_many_classes_without_register_tiles": {18: 0},
+    "nd_many_classes_without_register_tiles_nontemporal": {18: 0, 17: 0, 5: 0},
 }
 
 
@@ -69,7 +73,9 @@ def test_softmax_under_tuning(tuned, oracle):
             T_sm.test_softmax_rows(oracle, name, K, R)
     T_sm.test_softmax_cat_nll_and_bwd_rows(oracle, 1000, 256)
     for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3), (16, 200, 2), (1024, 256, 2),
-                    (196, 70, 3), (100, 100, 3), (196, 150, 2), (64, 300, 3), (196, 200, 2), (256, 65, 2), (324, 70, 2)]:
+                    (196, 70, 3), (100, 100, 3), (196, 150, 2), (64, 300, 3), (196, 200, 2), (256, 65, 2), (324, 70, 2),
+                    (1028, 48, 2), (1032, 65, 2), (1028, 129, 1), (1024, 192, 1), (1056, 200, 2), (1028, 300, 1),
+                    (784, 100, 2), (2048, 472, 1), (900, 65, 1)]:
         T_sm.test_softmax_nd_all_symbols(oracle, P, C, N)
 
 
@@ -81,5 +87,5 @@ def test_additive_under_tuning(tuned, oracle):
     for masked in (False, True):
         T_add.test_fused_batch_norm_equals_the_launch_sequence(oracle, 784, 16, 32, masked)
     T_add.test_fused_softmax_nd_nll_equals_the_two_launches(oracle, 2048, 19, 2)
-    for P, C, N in [(196, 82, 2), (64, 300, 3), (196, 200, 2)]:
+    for P, C, N in [(196, 82, 2), (64, 300, 3), (196, 200, 2), (1056, 200, 1), (1028, 300, 1)]:
         T_add.test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N)
