@@ -1027,7 +1027,9 @@ __device__ inline float vrcp(float a) { return 1.0f / a; }
 __device__ inline f32x4 vrcp(f32x4 a) { return f32x4{1.0f / a.x, 1.0f / a.y, 1.0f / a.z, 1.0f / a.w}; }
 
 // Pixel-group geometry shared by the N-d kernels: group g covers pixels
-// [W*pg, W*pg + W) of sample n, with g = pg + groups_per_sample * n.
+// [W*pg, W*pg + W) of sample n, with g = pg + groups_per_sample * n.  Where W does not divide P, the last group of a
+// plane is moved back to end with the plane: it covers the plane's last W pixels, some of which the group before it
+// covers too (both compute and store the same values for those; the arrays must not alias, and P >= W).
 struct PixelGrid {
   uint32_t P, C, N;
   uint32_t total_groups;
@@ -1041,6 +1043,7 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
   pg.div_gps.divmod(g, q, r);
   n = q;
   p = r * uint32_t(W);
+  if (p + uint32_t(W) > pg.P) p = pg.P - uint32_t(W);
 }
 
 
@@ -1500,7 +1503,7 @@ PixelGrid make_pixel_grid(uint32_t P, uint32_t C, uint32_t N, int W, bool ignore
   pg.P = P;
   pg.C = C;
   pg.N = N;
-  const uint32_t gps = P / uint32_t(W);
+  const uint32_t gps = (P + uint32_t(W) - 1u) / uint32_t(W);
   pg.total_groups = gps * N;
   pg.div_gps = FastDiv(gps ? gps : 1);
   return pg;
@@ -1524,7 +1527,9 @@ void launch_softmax_nd_reg_nt(uint32_t P, uint32_t C, uint32_t N, const float *x
                               bool ignore = false) {
   // (the same lanes per group in every variant: the order of a pixel's sum, hence the bits of p, depends on it)
   PixelGrid pg = make_pixel_grid(P, C, N, PixVec<V>::W, ignore);
-  pg.xcd = (tuning().nd_xcd_mask & 1) ? 1u : 0u;
+  // (planes that are not whole 16-byte groups: neighbouring blocks, which write parts of the same lines, on one XCD:
+  // [4225, 19] 4.9 -> 5.2 TB/s, [1025, 4] 5.3 -> 5.8, [89401, 2] 5.1 -> 5.9; [65535, 32] loses, 4.7 -> 4.3)
+  pg.xcd = ((tuning().nd_xcd_mask & 1) || P % uint32_t(PixVec<V>::W) != 0) ? 1u : 0u;
   if constexpr (PixVec<V>::W == 4) {
     // more classes: eight lanes per pixel group, 8, 16 or 32 sixteen-byte values per lane
     if (C > 192) {
@@ -2211,7 +2216,7 @@ void launch_softmax_nd_samplereg(const SampleReg &sr, uint32_t P, uint32_t C, ui
 // whole 128-byte lines, with neighbouring tiles on one XCD so that the lines they share are fetched once:
 // [900, 100] 3.9 -> 5.6, [900, 200] 3.1 -> 5.3, [1028, 64] 4.0 -> 5.6, [676, 128] 3.8 -> 5.5.
 template <int NS, int THREADS, bool NLL, bool BWD, int NT>
-__global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4, uint32_t C, uint32_t Gt, uint32_t PH,
+__global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P, uint32_t C, uint32_t Gt, uint32_t PH,
                                                                    uint32_t total_tiles, FastDiv div_gt,
                                                                    FastDiv div_tiles, uint32_t ignore, uint32_t xcd,
                                                                    const float *__restrict__ x, float *__restrict__ y,
@@ -2229,12 +2234,15 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4,
     const uint32_t b = (xcd && gridDim.x == total_tiles) ? xcd_contiguous(b0, total_tiles) : b0;
     uint32_t n, ti;
     div_tiles.divmod(b, n, ti);
+    const uint32_t P4 = (P + 3u) / 4u;  // pixel groups of a plane; the last one ends with the plane (PixelGrid)
     const uint32_t g0 = ti * Gt;
     const uint32_t gt = P4 - g0 < Gt ? P4 - g0 : Gt;
     const bool live = phase < PH && g < gt;
-    const size_t first = size_t(n) * C * P4 + g0 + g;  // in 16-byte groups: class c of this thread's pixels is c * P4 further
-    const f32x4 *xs = reinterpret_cast<const f32x4 *>(x) + first;
-    const size_t pix = (size_t(n) * P4 + g0 + g) * 4u;
+    uint32_t p = 4u * (g0 + g);
+    if (p + 4u > P) p = P - 4u;
+    const size_t first = size_t(n) * C * P + p;  // class c of this thread's pixels is c * P further
+    const float *xs = x + first;
+    const size_t pix = size_t(n) * P + p;
     u32x4 lab = {0u, 0u, 0u, 0u};
     f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
     if (NLL && live) lab = load_stream<0>(reinterpret_cast<const u32x4 *>(cat + pix));
@@ -2243,7 +2251,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4,
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
       const uint32_t c = uint32_t(i) * PH + phase;
-      v[i] = (live && c < C) ? load_stream<NT>(xs + size_t(c) * P4) : ninf;
+      v[i] = (live && c < C) ? load_stream<NT>(reinterpret_cast<const f32x4 *>(xs + size_t(c) * P)) : ninf;
     }
     f32x4 m = ninf;
 #pragma unroll
@@ -2273,14 +2281,14 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4,
           if (lab[w] >= C) d[w] = 0.0f;
         }
       }
-      f32x4 *ys = reinterpret_cast<f32x4 *>(y) + first;
-      f32x4 *ds = BWD ? reinterpret_cast<f32x4 *>(dx) + first : nullptr;
+      float *ys = y + first;
+      float *ds = BWD ? dx + first : nullptr;
 #pragma unroll
       for (int i = 0; i < NS; ++i) {
         const uint32_t c = uint32_t(i) * PH + phase;
         if (c < C) {
           const f32x4 pr = v[i] * inv;
-          store_stream<NT>(ys + size_t(c) * P4, pr);
+          store_stream<NT>(reinterpret_cast<f32x4 *>(ys + size_t(c) * P), pr);
           if (NLL) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
@@ -2291,7 +2299,7 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4,
             f32x4 gr;
 #pragma unroll
             for (int w = 0; w < 4; ++w) gr[w] = d[w] * (pr[w] - float(lab[w] == c));
-            store_stream<NT>(ds + size_t(c) * P4, gr);
+            store_stream<NT>(reinterpret_cast<f32x4 *>(ds + size_t(c) * P), gr);
           }
         }
       }
@@ -2316,9 +2324,9 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P4,
 ColReg nd_col_reg(uint32_t P, uint32_t C) {
   ColReg cr = {0, 0, 0, 0, 0, false};
   if (tuning().nd_colreg == 0) return cr;
-  if (P % 4u != 0 || P < 128u || C <= 32u || C > 512u) return cr;
-  const uint32_t P4 = P / 4u;
-  const bool lines = P4 % 8u == 0;
+  if (P < 128u || C <= 32u || C > 512u) return cr;
+  const uint32_t P4 = (P + 3u) / 4u;  // (planes that are not whole 16-byte groups: the last group ends with the plane)
+  const bool lines = P % 32u == 0;
   const uint32_t ns = (C <= 128u || (!lines && C <= 256u)) ? 8u : 16u;
   const uint32_t ph_need = (C + ns - 1u) / ns;  // at most 32
   const uint32_t step = lines ? 8u : 4u;
@@ -2348,6 +2356,8 @@ ColReg nd_col_reg(uint32_t P, uint32_t C) {
   cr.Gt = Gt;
   cr.PH = PH;
   cr.tiles = (P4 + Gt - 1u) / Gt;
+  // (planes that are not whole lines: neighbouring tiles, which share lines, on one XCD -- [16385, 100] 3.8 -> 5.3 TB/s,
+  // [4225, 150] 3.9 -> 4.9; one shape measured loses, [65535, 64] 4.8 -> 3.8)
   cr.xcd = lines ? 0u : 1u;
   cr.fits = true;
   return cr;
@@ -2357,7 +2367,6 @@ template <bool NLL, bool BWD>
 void launch_softmax_nd_colreg(const ColReg &cr, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                               const uint32_t *cat, float *nll, const float *dy, float *dx, bool ignore,
                               hipStream_t s) {
-  const uint32_t P4 = P / 4u;
   const uint64_t total = uint64_t(cr.tiles) * N;  // at most len / 128: a tile is 33 classes of 4 pixel groups or more
   uint32_t max_blocks = 1u << 24;
   if (tuning().flat_wg_per_cu > 0) max_blocks = uint32_t(device_cu_count()) * uint32_t(tuning().flat_wg_per_cu);  // (the tests' way into the loop over tiles)
@@ -2371,10 +2380,10 @@ void launch_softmax_nd_colreg(const ColReg &cr, uint32_t P, uint32_t C, uint32_t
     constexpr int NT = decltype(policy)::value;
     if (cr.ns == 8) {
       softmax_nd_colreg_kernel<8, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
-          P4, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
+          P, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
     } else {
       softmax_nd_colreg_kernel<16, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
-          P4, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
+          P, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
     }
   });
 }
@@ -2389,6 +2398,12 @@ bool nd_one_pixel_per_thread(uint32_t P, uint32_t C, bool vec) { return (!vec ||
 // does not matter (the accesses only ask for 4-byte alignment), so every entry point picks the same kernel family
 // for a shape and a pixel's sum is added in the same order by all of them
 bool nd_vec(uint32_t P) { return P % 4 == 0; }
+
+// Planes that are not whole 16-byte groups, up to 32 classes: the two-lane kernel over groups of four pixels all the
+// same, 16-byte accesses at 4-byte-aligned addresses, the last group of a plane moved back to end with the plane
+// (PixelGrid).  Against one pixel per thread: [4225, 2] 4.5 -> 5.8 TB/s, [1025, 4] 4.9 -> 5.8, [4225, 19] 5.0 -> 5.2,
+// [263169, 21] 4.3 -> 4.9 (what is left to the aligned rate, 6.0, is the stores that straddle 16-byte groups).
+bool nd_overlapped_pairs(uint32_t P, uint32_t C) { return P % 4 != 0 && P >= 8 && C <= 32; }
 
 void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                        CUstream_st *stream) {
@@ -2406,7 +2421,7 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     launch_softmax_nd_samplereg<false, false>(sr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (nd_tile_fits(P, C)) {
     launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
-  } else if (const ColReg cr = nd_col_reg(P, C); cr.fits) {
+  } else if (const ColReg cr = nd_col_reg(P, C); cr.fits && (vec || x != y)) {
     launch_softmax_nd_colreg<false, false>(cr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
   } else if (vec && ct.fits) {
     launch_softmax_nd_coltile<false, false>(ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
@@ -2420,7 +2435,7 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     } else {
       softmax_nd_reg_kernel<128, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
     }
-  } else if (vec) {
+  } else if (vec || (nd_overlapped_pairs(P, C) && x != y)) {
     launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
   } else {
     launch_softmax_nd_typed<float>(P, C, N, x, y, s);
@@ -2648,7 +2663,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
     launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                         as_stream(stream));
     note_launch(__func__);
-  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits) {
+  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits && (nd_vec(prefix_dim) || x != softmax)) {
     launch_softmax_nd_colreg<true, false>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
                                           as_stream(stream));
     note_launch(__func__);
@@ -2661,7 +2676,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_
              // plain entry point)
              dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
-    if (vec) {
+    if (vec || (nd_overlapped_pairs(prefix_dim, dim0) && x != softmax)) {
       launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
     } else {
       launch_softmax_nd_reg<float, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
@@ -2694,7 +2709,8 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
     launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                        as_stream(stream));
     note_launch(__func__);
-  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits) {
+  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0);
+             cr.fits && (nd_vec(prefix_dim) || (x != softmax && x != dx))) {
     launch_softmax_nd_colreg<true, true>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
                                          as_stream(stream));
     note_launch(__func__);
@@ -2706,7 +2722,7 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
   } else if (const bool vec = nd_vec(prefix_dim);
              dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
     hipStream_t s = as_stream(stream);
-    if (vec) {
+    if (vec || (nd_overlapped_pairs(prefix_dim, dim0) && x != softmax && x != dx)) {
       launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
     } else {
       launch_softmax_nd_reg<float, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);

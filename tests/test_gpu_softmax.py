@@ -268,6 +268,11 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # slots per thread, ragged last tiles, planes that are and are not whole 128-byte lines
              (128, 33, 3), (124, 300, 2), (132, 512, 2), (1028, 513, 1), (900, 300, 1), (400, 200, 2), (4100, 40, 1),
              (2048, 257, 1), (1024, 512, 1), (324, 256, 2), (4096, 64, 1),
+             # planes that are not whole 16-byte groups through the 16-byte kernels (the last group of a plane ends
+             # with the plane): two lanes per group up to 32 classes where no LDS tile holds the sample, column tiles
+             # in registers from 129 pixels on
+             (1001, 19, 2), (1023, 9, 2), (2049, 2, 3), (4225, 21, 1), (1026, 32, 2), (129, 33, 3), (131, 512, 1),
+             (4225, 64, 1), (1031, 300, 1),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
@@ -309,7 +314,7 @@ def test_softmax_nd_all_symbols(oracle, P, C, N):
 
 @pytest.mark.parametrize("P,C,N", [(64, 19, 3), (196, 19, 5), (196, 70, 3), (64, 300, 2), (1056, 200, 1), (2048, 19, 2),
                                    (1028, 300, 1), (36, 128, 3), (196, 150, 2), (400, 40, 2), (784, 40, 1), (196, 200, 2), (900, 65, 1), (900, 300, 1),
-                                   (2048, 257, 1)])
+                                   (2048, 257, 1), (1001, 19, 2), (1025, 100, 1)])
 def test_softmax_nd_arrays_that_lie_differently(oracle, P, C, N):
     # every n-d kernel family with arrays at different element offsets from a 16-byte boundary: the 16-byte forms
     # need all of a launch's arrays aligned, and any mix must still give the 4-byte forms' (correct) results;
@@ -422,3 +427,20 @@ def test_softmax_nd_special_values(oracle, C, P):
         assert np.all(np.isnan(p[0, :, 2])) and np.all(np.isnan(p[1, :, 6]))
         assert not np.any(np.isnan(np.delete(p.reshape(N * C, P), [2], axis=1)[:C]))
         assert np.all(p[0, :, 3] == p[0, 0, 3]) and abs(float(p[0, 0, 3]) * C - 1) < 1e-6
+
+
+@pytest.mark.parametrize("P,C,N", [(64, 19, 3), (1025, 19, 2), (1025, 100, 1), (1028, 100, 1), (196, 100, 2), (7, 9, 50),
+                                   (2049, 2, 2), (400, 300, 1)])
+def test_softmax_nd_in_place(oracle, P, C, N):
+    # y == x, as the reference's kernels allow (a thread reads nothing but the pixels it writes).  Planes that are
+    # not whole 16-byte groups then keep their kernels with one pixel per thread: the 16-byte kernels let the last
+    # two groups of such a plane overlap, which needs separate arrays.
+    g = np.random.default_rng(P + C)
+    n = P * C * N
+    x = g.standard_normal(n).astype(F32)
+    want = oracle.softmax_nd(P, C, N, x, f64=True)
+    for offset in (0, 1):
+        xd = dev(x, offset)
+        call("anode_gpu_softmax_nd_packed_f32", P, C, N, xd, xd)
+        assert_close(host(xd), want, "softmax_nd in place", abs_floor=1e-30)
+
