@@ -1662,6 +1662,12 @@ constexpr uint32_t kNdTileMaxSample = 8192;    // a larger sample has a tile to 
 constexpr uint32_t kNdTileBigSample = 16128;   // ... and up to 63 KB from 33 classes on, where nothing else fits
 bool nd_tile_fits(uint32_t P, uint32_t C);
 
+struct ColReg {  // the tiling of softmax_nd_colreg_kernel, further down
+  uint32_t ns, Gt, PH, tiles, xcd;
+  bool fits;
+};
+ColReg nd_col_reg(uint32_t P, uint32_t C);
+
 template <bool NLL, bool BWD, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uint32_t C, uint32_t N, uint32_t SB,
                                                                  FastDiv div_p, FastDiv div_c, int vec, uint32_t ignore,
@@ -1676,7 +1682,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_tile_kernel(uint32_t P, uin
   for (uint64_t n0 = uint64_t(blockIdx.x) * SB; n0 < N; n0 += uint64_t(gridDim.x) * SB) {
     const uint32_t samples = (N - n0 < uint64_t(SB)) ? uint32_t(N - n0) : SB;
     const uint32_t n = samples * slab;
-    const uint32_t n4 = vec ? n / 4u : 0u;  // (the host checked that every tile starts a whole number of 16-byte groups into the array)
+    const uint32_t n4 = vec ? n / 4u : 0u;  // (16-byte copies; what is left of the tile goes element by element)
     const float *xt = x + n0 * slab;
     float *yt = y + n0 * slab;
     // eight groups per thread are requested before the first is written to LDS (a slot past the tile's end reads
@@ -1781,12 +1787,14 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
   uint32_t blocks = (N + SB - 1u) / SB;
   const uint32_t max_blocks = 1u << 24;
   if (blocks > max_blocks) blocks = max_blocks;
-  const bool starts_aligned = (uint64_t(SB) * slab) % 4u == 0 || N <= SB;
-  const int vec = starts_aligned ? 1 : 0;  // (tiles of whole 16-byte groups, wherever the arrays lie)
+  // 16-byte copies between the arrays and the tile wherever the tiles start (4-byte-aligned accesses; with 4-byte
+  // copies for tiles that do not start a whole number of groups into the array, [169, 19] ran at 3.5 TB/s)
+  const int vec = 1;
+  const bool whole_pieces = (uint64_t(SB) * slab) % 16u == 0 || N <= SB;  // every tile starts on a 64-byte boundary if the arrays do
   const size_t lds_bytes = size_t(SB) * slab * sizeof(float);
   const FastDiv div_p(P), div_c(C);
   // logits in, probabilities (and the gradient) out: all streamed
-  const int nt = policy_for_outputs(stream_policy(size_t(slab) * N * sizeof(float), tuning().nontemporal), y, dx);
+  const int nt = whole_pieces ? policy_for_outputs(stream_policy(size_t(slab) * N * sizeof(float), tuning().nontemporal), y, dx) : 0;
   with_stream_policy(nt, [&](auto policy) {
     softmax_nd_tile_kernel<NLL, BWD, decltype(policy)::value>
         <<<blocks, kBlock, lds_bytes, s>>>(P, C, N, SB, div_p, div_c, vec, ignore ? 1u : 0u, x, y, cat, nll, dy, dx);
@@ -1860,6 +1868,8 @@ bool nd_tile_fits(uint32_t P, uint32_t C) {
   const uint64_t sample = uint64_t(P) * C;
   if (C <= 64 && sample <= kNdTileMaxSample) return true;
   if (C > 32 && sample <= kNdTileBigSample) {
+    // (from 128 pixels on, column tiles in registers: [169, 64] 4.3 TB/s through a tile of one sample, 5.5 through them; [225, 64] 3.8 -> 5.4)
+    if (nd_col_reg(P, C).fits) return false;
     const ColTile ct = nd_col_tile(P, C);
     return !(ct.fits && ct.L >= 2);  // several threads per pixel over whole planes are faster
   }
@@ -2021,12 +2031,6 @@ void launch_softmax_nd_coltile(const ColTile &ct, uint32_t P, uint32_t C, uint32
 // the sample: every access is 16 bytes per lane over whole runs of the array, whatever P is, x is read once, and
 // nothing but the PH partial maxima and sums of a pixel group goes through LDS.  A pixel's sum is the sum of its PH
 // partial sums in phase order, each added in class order: it depends on the shape and on nothing else.
-struct ColReg {  // the tiling of softmax_nd_colreg_kernel, further down
-  uint32_t ns, Gt, PH, tiles, xcd;
-  bool fits;
-};
-ColReg nd_col_reg(uint32_t P, uint32_t C);
-
 struct SampleReg {
   uint32_t threads;  // 256, 512 or 1024: the kernel's launch bound
   uint32_t ns;       // 8 or 16 slots per thread

@@ -479,7 +479,7 @@ def shape_sweep(torch, gpu):
             "K": K, "R": R,
             "softmax_packed_block": rate(lambda i: gpu.call("anode_gpu_softmax_packed_block_f32", K, R, x[i % 3],
                                                             x[3 + i % 3]), 8 * n)})
-    for P in (65536, 400, 196):
+    for P in (65536, 4225, 400, 196):
         for C in (2, 4, 19, 32, 33, 64, 100, 128, 150, 256, 300):
             N = min(total // (P * C), 1 << 20)
             if N < 1:
