@@ -2514,6 +2514,60 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_kernel(uin
   }
 }
 
+// The flat walk for planes that are not whole 16-byte groups: a thread still takes one 16-byte group of dx, which now
+// may lie across the end of a plane (its pixels then belong to two classes, or to two samples) or across the end of
+// the array.  A group inside one plane fetches dy and labels with 16-byte accesses at 4-byte-aligned addresses; the
+// one group per plane that lies across its end, and the array's last group, go element by element.  The stores stay
+// aligned 16-byte ones, which the kernels with one pixel per thread do not have: [4225, 19] 4.3 -> 5.0 TB/s,
+// [1025, 100] 3.2 -> 5.1, [961, 64] 4.0 -> 5.1, [65535, 4] 4.2 -> 5.1.
+template <bool ACC, int NT>
+__global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_any_kernel(uint32_t P, uint32_t C, uint32_t len,
+                                                                                 FastDiv div_p, FastDiv div_c,
+                                                                                 uint32_t ignore,
+                                                                                 const float *__restrict__ dy,
+                                                                                 const float *__restrict__ prob,
+                                                                                 const uint32_t *__restrict__ cat,
+                                                                                 float *dx) {
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
+  const uint32_t total_groups = (len + 3u) / 4u;
+  for (uint64_t g64 = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g64 < total_groups; g64 += stride) {
+    const uint32_t e = uint32_t(g64) * 4u;  // the group's first element
+    uint32_t plane, r;                      // plane = n * C + k, r = the pixel
+    div_p.divmod(e, plane, r);
+    if (r + 4u <= P && e + 4u <= len) {
+      const uint32_t n = div_c.div(plane);
+      const uint32_t k = plane - n * C;
+      const size_t pix = size_t(n) * P + r;
+      f32x4 d = load_stream<0>(reinterpret_cast<const f32x4 *>(dy + pix));
+      const u32x4 lab = load_stream<0>(reinterpret_cast<const u32x4 *>(cat + pix));
+      const f32x4 pr = load_stream<NT>(reinterpret_cast<const f32x4 *>(prob + e));
+      f32x4 old = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (ACC) old = load_stream<NT>(reinterpret_cast<const f32x4 *>(dx + e));
+      f32x4 out;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        if (ignore && lab[w] >= C) d[w] = 0.0f;
+        const float t = pr[w] - float(lab[w] == k);
+        out[w] = ACC ? fmaf(d[w], t, old[w]) : d[w] * t;
+      }
+      store_stream<NT>(reinterpret_cast<f32x4 *>(dx + e), out);
+    } else {
+      for (uint32_t w = 0; w < 4u && e + w < len; ++w) {
+        uint32_t pl, rr;
+        div_p.divmod(e + w, pl, rr);
+        const uint32_t n = div_c.div(pl);
+        const uint32_t k = pl - n * C;
+        const size_t pix = size_t(n) * P + rr;
+        const uint32_t label = cat[pix];
+        float d = dy[pix];
+        if (ignore && label >= C) d = 0.0f;
+        const float t = prob[e + w] - float(label == k);
+        dx[e + w] = ACC ? fmaf(d, t, dx[e + w]) : d * t;
+      }
+    }
+  }
+}
+
 // The backward pass is a map, so with few pixels and many classes the classes are shared out as well: runs of
 // `chunk` classes (a multiple of 16: a thread reads its pixels' dy and labels once per run) over blockIdx.y, as
 // many as it takes to give the GPU eight workgroups per CU ([65536, 256, 4]: 256 workgroups of pixel groups).
@@ -2548,6 +2602,15 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
       softmax_nd_cat_nll_bwd_flat_kernel<ACC, decltype(policy)::value>
           <<<stream_grid(total_groups, 1), kBlock, 0, s>>>(P, C, total_groups, div_gpp, div_c, ignore ? 1u : 0u, dy, prob,
                                                           cat, dx);
+    });
+  } else if (!vec && P >= 512 && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
+    // (shorter planes: a wave of 256 elements then always holds a group that lies across the end of a plane and
+    // walks it element by element, [169, 19] accumulating 4.7 TB/s with one pixel per thread against 3.4 here)
+    const FastDiv div_p(P), div_c(C);
+    with_stream_policy(policy_for_outputs(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), dx), [&](auto policy) {
+      softmax_nd_cat_nll_bwd_flat_any_kernel<ACC, decltype(policy)::value>
+          <<<stream_grid((uint64_t(len) + 3u) / 4u, 1), kBlock, 0, s>>>(P, C, len, div_p, div_c, ignore ? 1u : 0u, dy, prob,
+                                                                       cat, dx);
     });
   } else if (vec) {
     PixelGrid pg = make_pixel_grid(P, C, N, 4, ignore);

@@ -168,7 +168,8 @@ def test_row_nll_ignore(K, R):
     assert_bit_exact(host(dx).reshape(R, K)[~keep], old.reshape(R, K)[~keep], "ignored rows untouched")
 
 
-@pytest.mark.parametrize("P,C,N", [(64, 19, 2), (37, 5, 3), (1, 10, 8), (4096, 19, 2), (8, 70, 2)])
+@pytest.mark.parametrize("P,C,N", [(64, 19, 2), (37, 5, 3), (1, 10, 8), (4096, 19, 2), (8, 70, 2), (1025, 7, 2),
+                                   (515, 3, 3)])
 def test_nd_nll_ignore(P, C, N):
     g = np.random.default_rng(P * C + N)
     p = oracle.softmax_nd(P, C, N, g.standard_normal(P * C * N).astype(F32))

@@ -75,7 +75,7 @@ def test_softmax_under_tuning(tuned, oracle):
     for P, C, N in [(2048, 19, 2), (1300, 19, 3), (8, 64, 3), (7, 40, 3), (16, 200, 2), (1024, 256, 2),
                     (196, 70, 3), (100, 100, 3), (196, 150, 2), (64, 300, 3), (196, 200, 2), (256, 65, 2), (324, 70, 2),
                     (1028, 48, 2), (1032, 65, 2), (1028, 129, 1), (1024, 192, 1), (1056, 200, 2), (1028, 300, 1),
-                    (784, 100, 2), (2048, 472, 1), (900, 65, 1)]:
+                    (784, 100, 2), (2048, 472, 1), (900, 65, 1), (1025, 19, 2), (515, 40, 2)]:
         T_sm.test_softmax_nd_all_symbols(oracle, P, C, N)
 
 
