@@ -1790,7 +1790,9 @@ void launch_softmax_nd_tile(uint32_t P, uint32_t C, uint32_t N, const float *x, 
   // 16-byte copies between the arrays and the tile wherever the tiles start (4-byte-aligned accesses; with 4-byte
   // copies for tiles that do not start a whole number of groups into the array, [169, 19] ran at 3.5 TB/s)
   const int vec = 1;
-  const bool whole_pieces = (uint64_t(SB) * slab) % 16u == 0 || N <= SB;  // every tile starts on a 64-byte boundary if the arrays do
+  // streaming stores where every tile starts a whole number of 16-byte groups into the array: the copy steps of a
+  // wave then cover whole lines of the array wherever the tile starts ([196, 19] 5.5 TB/s with ordinary stores, 6.0)
+  const bool whole_pieces = (uint64_t(SB) * slab) % 4u == 0 || N <= SB;
   const size_t lds_bytes = size_t(SB) * slab * sizeof(float);
   const FastDiv div_p(P), div_c(C);
   // logits in, probabilities (and the gradient) out: all streamed

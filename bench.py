@@ -73,8 +73,8 @@ MEASURED_TRAFFIC = {
     ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): (308434067, "bn_maps"),
     ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): (1610547205, "flat_maps"),
     ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): (637597563, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291356156, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671292527, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291319296, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671286383, "softmax"),
     ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): (192699228, "flat_maps"),
     ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): (192703324, "flat_maps"),
 }
@@ -89,10 +89,10 @@ TRAFFIC_FAMILY_SOURCES = {
     "softmax": ["common.hpp", "softmax.hip"],
 }
 TRAFFIC_FAMILY_FINGERPRINT = {
-    "bn_maps": "4d02d8d7280b081e",
-    "bn_reductions": "10f7ba7330302d99",
-    "flat_maps": "c6691b9dd66bc786",
-    "softmax": "09817018d533cf9e",
+    "bn_maps": "9d94a1d3c0e0f479",
+    "bn_reductions": "e27eb3a6158f909f",
+    "flat_maps": "c8b36a639e6d43e9",
+    "softmax": "a0ccfd781fbb6782",
 }
 
 

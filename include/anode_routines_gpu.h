@@ -167,7 +167,8 @@ void anode_gpu_softmax_cat_nll_packed_f32(uint32_t dim0, uint32_t dim1, const fl
 void anode_gpu_softmax_cat_nll_bwd_packed_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
 /* lib.h:465-473, softmax.cu:212-225.  dx += ... */
 void anode_gpu_softmax_cat_nll_bwd_packed_accumulate_f32(uint32_t dim0, uint32_t dim1, const float *dy, const float *softmax, const uint32_t *cat_data, float *dx, ANODE_LAUNCH_TAIL);
-/* lib.h:474-481, softmax.cu:227-276.  Channel-axis softmax per pixel. */
+/* lib.h:474-481, softmax.cu:227-276.  Channel-axis softmax per pixel.  y may be x (in place), as with the
+ * reference's kernel, whose threads read nothing but the pixels they write. */
 void anode_gpu_softmax_nd_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *x, float *y, ANODE_LAUNCH_TAIL);
 /* lib.h:482-490, softmax.cu:278-313.  Per-pixel gather, NaN when label >= dim0. */
 void anode_gpu_softmax_nd_cat_nll_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1, const float *softmax, const uint32_t *cat_data, float *nll, ANODE_LAUNCH_TAIL);
