@@ -550,6 +550,14 @@ constexpr size_t kNoAllocScratchBytes = size_t(4) << 20;  // 4 MiB per GPU, held
 constexpr int kNoAllocMaxDevices = 64;
 std::mutex g_noalloc_mutex;
 void *g_noalloc_ptr[kNoAllocMaxDevices] = {};  // device address of `scratch` on each GPU, looked up once
+// Calls on different streams of one GPU share that GPU's array.  Outside graph capture they are put in order on the
+// device: every call records this event behind its kernels, and a call on another stream than the last one waits for
+// it first.  The event is created with the address look-up, once per device; the mutex is held from the wait to the
+// record, so host threads cannot interleave their calls.
+std::mutex g_noalloc_order_mutex;
+hipEvent_t g_noalloc_done[kNoAllocMaxDevices] = {};
+hipStream_t g_noalloc_last_stream[kNoAllocMaxDevices] = {};
+bool g_noalloc_recorded[kNoAllocMaxDevices] = {};
 }  // namespace
 
 static __device__ __align__(256) double scratch[kNoAllocScratchBytes / sizeof(double)];
@@ -570,6 +578,13 @@ static void *noalloc_scratch_of_current_device(const char *symbol) {
       note_error(symbol, e != hipSuccess ? e : hipErrorInvalidSymbol, "cannot look up the scratch array");
       return nullptr;
     }
+    hipEvent_t done = nullptr;
+    const hipError_t ee = hipEventCreateWithFlags(&done, hipEventDisableTiming);
+    if (ee != hipSuccess || !done) {
+      note_error(symbol, ee != hipSuccess ? ee : hipErrorUnknown, "cannot create the event that orders calls on the scratch array");
+      return nullptr;
+    }
+    g_noalloc_done[dev] = done;
     g_noalloc_ptr[dev] = p;
   }
   return g_noalloc_ptr[dev];
@@ -594,15 +609,40 @@ ANODE_EXPORT int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, 
     return kReduceScratchTooSmall;
   }
   FixedScratch fixed{nullptr, kNoAllocScratchBytes};
-  if (need > 0) {
-    fixed.ptr = noalloc_scratch_of_current_device(__func__);
-    if (!fixed.ptr) return kReduceScratchUnavailable;
+  const MeanVarReduce op{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)};
+  if (need == 0) return launch_chan_reduce(__func__, dim0, dim1, dim2, op, x, nullptr, stream, nullptr, &fixed);
+  fixed.ptr = noalloc_scratch_of_current_device(__func__);
+  if (!fixed.ptr) return kReduceScratchUnavailable;
+  int dev = 0;
+  (void)hipGetDevice(&dev);  // (checked by the look-up above)
+  hipStream_t s = as_stream(stream);
+  std::lock_guard<std::mutex> order(g_noalloc_order_mutex);
+  // A stream under capture takes no part in the ordering: an event recorded into a capture cannot be waited for
+  // from outside it, and a captured call runs whenever its graph is launched.  Such callers keep their calls on one
+  // GPU from overlapping themselves.  (A capture state that cannot be read counts as capturing.)
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  const bool plain = hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
+  if (!plain) (void)hipGetLastError();
+  if (plain && g_noalloc_recorded[dev] && g_noalloc_last_stream[dev] != s) {
+    const hipError_t w = hipStreamWaitEvent(s, g_noalloc_done[dev], 0);
+    if (w != hipSuccess) {
+      note_error(__func__, w, "cannot wait for the previous call on the scratch array; nothing was enqueued");
+      return kReduceScratchUnavailable;
+    }
   }
   // Every partial that the second kernel reads is written by the first kernel of the same call, so nothing in
   // the array has to start at zero.
-  return launch_chan_reduce(__func__, dim0, dim1, dim2,
-                            MeanVarReduce{x, mean, var, dim0, double(dim0) * double(dim2), double(epsilon)}, x, nullptr,
-                            stream, nullptr, &fixed);
+  const int rc = launch_chan_reduce(__func__, dim0, dim1, dim2, op, x, nullptr, stream, nullptr, &fixed);
+  if (plain) {
+    const hipError_t r = hipEventRecord(g_noalloc_done[dev], s);
+    if (r == hipSuccess) {
+      g_noalloc_last_stream[dev] = s;
+      g_noalloc_recorded[dev] = true;
+    } else {
+      note_error(__func__, r, "cannot record the event that orders calls on the scratch array");
+    }
+  }
+  return rc;
 }
 
 ANODE_EXPORT void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2,

@@ -229,9 +229,12 @@ void anode_gpu_batch_mean_var_online_3d1_packed_f32(uint32_t dim0, uint32_t dim1
  * go to a 4 MiB device array that is part of the library image (one copy per GPU, held until the process ends)
  * instead of the per-stream buffer: the call makes no hipMalloc / hipFree and no allocating library call.  Returns
  * 0, or non-zero with nothing enqueued: 1 = the shape needs more than 4 MiB of partial sums (2 * dim1 * tiles per
- * channel doubles; use the entry point above), 2 = the array's device address could not be obtained.  All calls on
- * one GPU share the array: calls that overlap on one GPU (two streams, two threads, two graphs replayed together)
- * race; calls in stream order on one stream do not. */
+ * channel doubles; use the entry point above), 2 = the array's device address could not be obtained, or the call
+ * could not be put in order behind the previous one.  All calls on one GPU share the array.  Outside graph capture
+ * the library keeps them apart on the device, whatever streams and host threads they come from: every call records an
+ * event behind its kernels (created once per device, with the address look-up), and a call on another stream than the
+ * previous one waits for it.  A call that is captured takes no part in that: graphs that hold such calls must not be
+ * replayed so that they overlap each other, or other calls of this entry point, on one GPU. */
 int anode_gpu_batch_mean_var_3d1_packed_noalloc_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, float epsilon, const float *x, float *mean, float *var, ANODE_LAUNCH_TAIL);
 /* batch_norm followed by positive_clip in one pass: t = (x-mean[c])*rsqrt(var[c]); y = t * float(t>0). */
 void anode_gpu_batch_norm_positive_clip_3d1_packed_f32(uint32_t dim0, uint32_t dim1, uint32_t dim2, const float *x, const float *mean, const float *var, float *y, ANODE_LAUNCH_TAIL);

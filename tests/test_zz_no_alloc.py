@@ -110,6 +110,36 @@ def test_stream_order_keeps_calls_apart():
         assert_bit_exact(host(v), host(rv), "var")
 
 
+def test_calls_on_two_streams_are_put_in_order():
+    # Calls on different streams of one GPU share the array; outside graph capture the library orders them on the
+    # device (each call waits for the event the previous call recorded behind its kernels), so neither stream's
+    # partial sums are overwritten while its second kernel still reads them.  Two streams, no host synchronisation
+    # in between, a long and a short reduction in turn, thirty rounds; every result against the allocating entry point.
+    big, small = (12544, 16, 32), (784, 16, 64)
+    g = np.random.default_rng(21)
+    xa = dev((1 + g.standard_normal(big[0] * big[1] * big[2])).astype(F32))
+    xb = dev((2 + g.standard_normal(small[0] * small[1] * small[2])).astype(F32))
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    rounds = 30
+    outs_a = [(empty(big[1]), empty(big[1])) for _ in range(rounds)]
+    outs_b = [(empty(small[1]), empty(small[1])) for _ in range(rounds)]
+    torch.cuda.synchronize()
+    for k in range(rounds):
+        assert _noalloc(*big, 1e-5, xa, *outs_a[k], stream=sa.cuda_stream) == 0
+        assert _noalloc(*small, 1e-5, xb, *outs_b[k], stream=sb.cuda_stream) == 0
+    sa.synchronize()
+    sb.synchronize()
+    ref_a, ref_b = (empty(big[1]), empty(big[1])), (empty(small[1]), empty(small[1]))
+    call(PLAIN, *big, 1e-5, xa, *ref_a)
+    call(PLAIN, *small, 1e-5, xb, *ref_b)
+    for k in range(rounds):
+        assert_bit_exact(host(outs_a[k][0]), host(ref_a[0]), f"mean, long reduction, round {k}")
+        assert_bit_exact(host(outs_a[k][1]), host(ref_a[1]), f"var, long reduction, round {k}")
+        assert_bit_exact(host(outs_b[k][0]), host(ref_b[0]), f"mean, short reduction, round {k}")
+        assert_bit_exact(host(outs_b[k][1]), host(ref_b[1]), f"var, short reduction, round {k}")
+
+
 def test_oversized_shape_is_refused():
     # With lane tiles switched off (tuning knob 9), [1, 65536, 4096] is cut into 32 sample tiles: 32 partials for
     # each of 65536 channels, two sums -> 32 MiB > 4 MiB.  The call must return 1 and enqueue nothing.  The buffers
