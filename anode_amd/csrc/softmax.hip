@@ -1043,7 +1043,7 @@ __device__ inline void pixel_decode(const PixelGrid &pg, uint32_t g, int W, uint
   pg.div_gps.divmod(g, q, r);
   n = q;
   p = r * uint32_t(W);
-  if (p + uint32_t(W) > pg.P) p = pg.P - uint32_t(W);
+  if (pg.P - p < uint32_t(W)) p = pg.P - uint32_t(W);  // (p < P)
 }
 
 
@@ -2531,12 +2531,12 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_any_kernel
                                                                                  const uint32_t *__restrict__ cat,
                                                                                  float *dx) {
   const uint64_t stride = uint64_t(gridDim.x) * kBlock;  // 64-bit: index + stride can pass 2^32
-  const uint32_t total_groups = (len + 3u) / 4u;
+  const uint64_t total_groups = (uint64_t(len) + 3u) / 4u;  // (64-bit: len + 3 can pass 2^32)
   for (uint64_t g64 = uint64_t(blockIdx.x) * kBlock + threadIdx.x; g64 < total_groups; g64 += stride) {
-    const uint32_t e = uint32_t(g64) * 4u;  // the group's first element
+    const uint32_t e = uint32_t(g64) * 4u;  // the group's first element: below len
     uint32_t plane, r;                      // plane = n * C + k, r = the pixel
     div_p.divmod(e, plane, r);
-    if (r + 4u <= P && e + 4u <= len) {
+    if (r + 4u <= P && uint64_t(e) + 4u <= len) {
       const uint32_t n = div_c.div(plane);
       const uint32_t k = plane - n * C;
       const size_t pix = size_t(n) * P + r;
@@ -2554,7 +2554,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_any_kernel
       }
       store_stream<NT>(reinterpret_cast<f32x4 *>(dx + e), out);
     } else {
-      for (uint32_t w = 0; w < 4u && e + w < len; ++w) {
+      for (uint32_t w = 0; w < 4u && uint64_t(e) + w < len; ++w) {
         uint32_t pl, rr;
         div_p.divmod(e + w, pl, rr);
         const uint32_t n = div_c.div(pl);

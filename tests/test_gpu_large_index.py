@@ -147,8 +147,43 @@ def test_softmax_nd_backward_beyond_2_31(big):
     del dx
 
 
+def test_softmax_nd_planes_that_are_not_whole_groups_beyond_2_31(big):
+    # planes of 65537 pixels: the 16-byte kernels over groups of four pixels whose last one ends with the plane (two
+    # lanes per group at 19 classes, column tiles in registers at 220), and the backward pass walked flat in dx's
+    # 16-byte groups wherever the planes end
+    for P, C, N in ((65537, 19, 1725), (65537, 220, 149)):
+        n = P * C * N
+        assert (1 << 31) < n <= N_BIG
+        x = big[:n]
+        p = torch.empty(n + 8, device="cuda")
+        p[n:] = 777.0
+        call("anode_gpu_softmax_nd_packed_f32", P, C, N, x, p[:n])
+        torch.cuda.synchronize()
+        assert bool((p[n:] == 777.0).all())
+        pv = p[:n].view(N, C, P)
+        for i in (0, N // 2, N - 1):
+            ref = torch.softmax(x.view(N, C, P)[i].double(), dim=0)
+            assert bool(((pv[i].double() - ref).abs() <= 1e-5 * ref).all()), (P, C, i)
+        sums = pv.sum(dim=1)
+        assert bool(((sums - 1).abs() < 1e-5).all())
+        del sums
+        lab = torch.randint(0, C + 1, (P * N,), device="cuda", dtype=torch.int32)
+        dy = torch.randn(P * N, device="cuda")
+        dx = torch.empty(n + 8, device="cuda")
+        dx[n:] = 555.0
+        call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dy, p[:n], lab, dx[:n])
+        torch.cuda.synchronize()
+        assert bool((dx[n:] == 555.0).all())
+        dv = dx[:n].view(N, C, P)
+        ks = torch.arange(C, device="cuda", dtype=torch.int32).view(C, 1)
+        for i in (0, N // 2, N - 1):
+            want = dy.view(N, P)[i].unsqueeze(0) * (pv[i] - (lab.view(N, P)[i].unsqueeze(0) == ks).float())
+            assert torch.equal(dv[i], want), (P, C, i)
+        del p, dx, lab, dy
+
+
 def test_softmax_nd_many_classes_beyond_2_31(big):
-    # 220 classes: tiles of all classes of 32 pixels in LDS
+    # 220 classes: column tiles in registers (a workgroup per run of 32 pixel groups with all their classes)
     P, C, N = 1 << 16, 220, 149          # 2 148 270 080 elements
     n = P * C * N
     assert (1 << 31) < n <= N_BIG
@@ -328,6 +363,28 @@ def test_batch_norm_pieces_close_to_2_32(huge):
         if yq is not None:                                 # the last channel ends at the last element of the array
             assert abs(yq - (1 - 1e-5 / v)) < 1e-4
     del y
+
+
+def test_softmax_nd_backward_over_odd_planes_close_to_2_32(huge):
+    # 4 294 574 085 elements in planes of 65535 pixels: the flat walk's last 16-byte group is a partial one, 2.7 * 10^5
+    # elements under 2^32
+    P, C, N = 65535, 19, 3449
+    n = P * C * N
+    assert (1 << 32) - (1 << 20) < n < (1 << 32) and n % 4 != 0
+    p = huge[:n]
+    lab = torch.randint(0, C, (P * N,), device="cuda", dtype=torch.int32)
+    dy = torch.randn(P * N, device="cuda")
+    dx = torch.empty(n + 8, device="cuda")
+    dx[n:] = 555.0
+    call("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", P, C, N, dy, p, lab, dx[:n])
+    torch.cuda.synchronize()
+    assert bool((dx[n:] == 555.0).all())
+    pv, dv = p.view(N, C, P), dx[:n].view(N, C, P)
+    ks = torch.arange(C, device="cuda", dtype=torch.int32).view(C, 1)
+    for i in (0, N // 2, N - 1):
+        want = dy.view(N, P)[i].unsqueeze(0) * (pv[i] - (lab.view(N, P)[i].unsqueeze(0) == ks).float())
+        assert torch.equal(dv[i], want), i
+    del dx, lab, dy
 
 
 def test_softmax_nd_close_to_2_32(huge):
