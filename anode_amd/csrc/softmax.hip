@@ -16,6 +16,7 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <cstring>
 
 namespace anode {
 namespace {
@@ -2411,6 +2412,62 @@ bool nd_vec(uint32_t P) { return P % 4 == 0; }
 // [263169, 21] 4.3 -> 4.9 (what is left to the aligned rate, 6.0, is the stores that straddle 16-byte groups).
 bool nd_overlapped_pairs(uint32_t P, uint32_t C) { return P % 4 != 0 && P >= 8 && C <= 32; }
 
+// Which kernel family a shape takes: one decision for the plain and the fused entry points, because the order in
+// which a pixel's exponentials are added, hence the bits of p, follows the kernel.  `separate` says that no output
+// array is the input array: planes that are not whole 16-byte groups need that for their 16-byte kernels, whose last
+// two groups of a plane overlap (with y == x such shapes take the kernels with one pixel per thread, whose sums are
+// added in another order; nothing else depends on the arrays).
+enum class NdFamily : uint32_t {
+  Rows = 0,        // P == 1
+  SampleReg = 1,   // whole samples in registers
+  Tile = 2,        // whole samples through an LDS tile
+  ColReg = 3,      // column tiles in registers
+  ColTile = 4,     // column tiles in LDS
+  PixelPerThread = 5,  // 33 to 128 classes, one pixel per thread (4-byte accesses)
+  Groups16 = 6,    // groups of four pixels: two lanes per group up to 32 classes, eight up to 256, two passes beyond
+  Singles = 7,     // single pixels: registers up to 32 classes, two passes beyond
+};
+struct NdPlan {
+  NdFamily family;
+  SampleReg sr;
+  ColReg cr;
+  ColTile ct;
+};
+
+NdPlan nd_plan(uint32_t P, uint32_t C, bool separate) {
+  NdPlan pl = {NdFamily::Singles, {0, 0, 0, 0, false}, {0, 0, 0, 0, 0, false}, {0, 0, 0, false}};
+  if (P == 1) {
+    pl.family = NdFamily::Rows;
+    return pl;
+  }
+  const bool vec = nd_vec(P);
+  pl.sr = nd_sample_reg(P, C);
+  if (pl.sr.fits) {
+    pl.family = NdFamily::SampleReg;
+    return pl;
+  }
+  if (nd_tile_fits(P, C)) {
+    pl.family = NdFamily::Tile;
+    return pl;
+  }
+  pl.cr = nd_col_reg(P, C);
+  if (pl.cr.fits && (vec || separate)) {
+    pl.family = NdFamily::ColReg;
+    return pl;
+  }
+  pl.ct = nd_col_tile(P, C);
+  if (vec && pl.ct.fits) {
+    pl.family = NdFamily::ColTile;
+    return pl;
+  }
+  if (nd_one_pixel_per_thread(P, C, vec)) {
+    pl.family = NdFamily::PixelPerThread;
+    return pl;
+  }
+  if (vec || (nd_overlapped_pairs(P, C) && separate)) pl.family = NdFamily::Groups16;
+  return pl;
+}
+
 void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x, float *y,
                        CUstream_st *stream) {
   const uint32_t len = checked_len(P, C, N, symbol);
@@ -2420,31 +2477,39 @@ void launch_softmax_nd(const char *symbol, uint32_t P, uint32_t C, uint32_t N, c
     return;
   }
   hipStream_t s = as_stream(stream);
-  const bool vec = nd_vec(P);
-  const ColTile ct = nd_col_tile(P, C);
-  const SampleReg sr = nd_sample_reg(P, C);
-  if (sr.fits) {
-    launch_softmax_nd_samplereg<false, false>(sr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
-  } else if (nd_tile_fits(P, C)) {
-    launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
-  } else if (const ColReg cr = nd_col_reg(P, C); cr.fits && (vec || x != y)) {
-    launch_softmax_nd_colreg<false, false>(cr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
-  } else if (vec && ct.fits) {
-    launch_softmax_nd_coltile<false, false>(ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
-  } else if (nd_one_pixel_per_thread(P, C, vec)) {
-    // one pixel per thread keeps
-    // the row in registers and is still coalesced across the wave
-    const PixelGrid pg = make_pixel_grid(P, C, N, 1);
-    const uint32_t blocks = pixel_blocks(pg.total_groups);
-    if (C <= 64) {
-      softmax_nd_reg_kernel<64, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
-    } else {
-      softmax_nd_reg_kernel<128, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+  const NdPlan pl = nd_plan(P, C, x != y);
+  switch (pl.family) {
+    case NdFamily::Rows:  // (taken above)
+      break;
+    case NdFamily::SampleReg:
+      launch_softmax_nd_samplereg<false, false>(pl.sr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+      break;
+    case NdFamily::Tile:
+      launch_softmax_nd_tile<false, false>(P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+      break;
+    case NdFamily::ColReg:
+      launch_softmax_nd_colreg<false, false>(pl.cr, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+      break;
+    case NdFamily::ColTile:
+      launch_softmax_nd_coltile<false, false>(pl.ct, P, C, N, x, y, nullptr, nullptr, nullptr, nullptr, false, s);
+      break;
+    case NdFamily::PixelPerThread: {
+      // one pixel per thread keeps the row in registers and is still coalesced across the wave
+      const PixelGrid pg = make_pixel_grid(P, C, N, 1);
+      const uint32_t blocks = pixel_blocks(pg.total_groups);
+      if (C <= 64) {
+        softmax_nd_reg_kernel<64, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      } else {
+        softmax_nd_reg_kernel<128, float, false, 0, 1><<<blocks, kBlock, 0, s>>>(pg, x, y, nullptr, nullptr);
+      }
+      break;
     }
-  } else if (vec || (nd_overlapped_pairs(P, C) && x != y)) {
-    launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
-  } else {
-    launch_softmax_nd_typed<float>(P, C, N, x, y, s);
+    case NdFamily::Groups16:
+      launch_softmax_nd_typed<f32x4>(P, C, N, x, y, s);
+      break;
+    case NdFamily::Singles:
+      launch_softmax_nd_typed<float>(P, C, N, x, y, s);
+      break;
   }
   note_launch(symbol);
 }
@@ -2714,48 +2779,68 @@ ANODE_EXPORT void anode_gpu_softmax_cat_nll_fused_fwd_bwd_packed_f32(uint32_t di
   launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
 }
 
+// The fused n-d entry points: the kernel that nd_plan() names for the shape, with the label gather (and the backward
+// pass) riding along; shapes whose kernel has no such form run the separate launches back to back.
+template <bool BWD>
+static void launch_softmax_nd_fused(const char *symbol, uint32_t P, uint32_t C, uint32_t N, const float *x,
+                                    const uint32_t *cat, const float *dy, float *softmax, float *nll, float *dx,
+                                    const KernelConfig *cfg, CUstream_st *stream) {
+  const uint32_t len = checked_len(P, C, N, symbol);
+  if (len == 0) return;
+  hipStream_t s = as_stream(stream);
+  const NdPlan pl = nd_plan(P, C, x != softmax && (!BWD || x != dx));
+  bool launched = true;
+  switch (pl.family) {
+    case NdFamily::Rows:  // the class axis is contiguous: the row form
+      launch_softmax_rows(symbol, C, N, x, softmax, stream, RowNll{cat, nll, false, BWD ? dy : nullptr, BWD ? dx : nullptr});
+      return;
+    case NdFamily::SampleReg:
+      launch_softmax_nd_samplereg<true, BWD>(pl.sr, P, C, N, x, softmax, cat, nll, dy, dx, false, s);
+      break;
+    case NdFamily::Tile:
+      launch_softmax_nd_tile<true, BWD>(P, C, N, x, softmax, cat, nll, dy, dx, false, s);
+      break;
+    case NdFamily::ColReg:
+      launch_softmax_nd_colreg<true, BWD>(pl.cr, P, C, N, x, softmax, cat, nll, dy, dx, false, s);
+      break;
+    case NdFamily::ColTile:
+      launch_softmax_nd_coltile<true, BWD>(pl.ct, P, C, N, x, softmax, cat, nll, dy, dx, false, s);
+      break;
+    case NdFamily::Groups16:
+      if (C <= 256) {
+        launch_softmax_nd_reg<f32x4, true, BWD>(P, C, N, x, softmax, cat, nll, s, dy, dx);
+      } else {
+        launched = false;
+      }
+      break;
+    case NdFamily::Singles:
+      if (C <= 32) {
+        launch_softmax_nd_reg<float, true, BWD>(P, C, N, x, softmax, cat, nll, s, dy, dx);
+      } else {
+        launched = false;
+      }
+      break;
+    case NdFamily::PixelPerThread:
+      launched = false;
+      break;
+  }
+  if (launched) {
+    note_launch(symbol);
+    return;
+  }
+  // shapes outside the kernels that carry the labels along: the separate passes, back to back
+  anode_gpu_softmax_nd_packed_f32(P, C, N, x, softmax, cfg, stream);
+  anode_gpu_softmax_nd_cat_nll_packed_f32(P, C, N, softmax, cat, nll, cfg, stream);
+  if (BWD) anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(P, C, N, dy, softmax, cat, dx, cfg, stream);
+}
+
 // Additive (no counterpart in the reference): softmax_nd and softmax_nd_cat_nll in one pass over x.
 // Writes the same probabilities and the same nll values as the two separate entry points.
 ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_packed_f32(uint32_t prefix_dim, uint32_t dim0, uint32_t dim1,
                                                                 const float *x, const uint32_t *cat_data,
                                                                 float *softmax, float *nll, const KernelConfig *cfg,
                                                                 CUstream_st *stream) {
-  const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
-  if (len == 0) return;
-  if (prefix_dim == 1) {  // the class axis is contiguous: the row form
-    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, nullptr, nullptr});
-  } else if (const SampleReg sr = nd_sample_reg(prefix_dim, dim0); sr.fits) {
-    launch_softmax_nd_samplereg<true, false>(sr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
-                                             false, as_stream(stream));
-    note_launch(__func__);
-  } else if (nd_tile_fits(prefix_dim, dim0)) {
-    launch_softmax_nd_tile<true, false>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
-                                        as_stream(stream));
-    note_launch(__func__);
-  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0); cr.fits && (nd_vec(prefix_dim) || x != softmax)) {
-    launch_softmax_nd_colreg<true, false>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr, false,
-                                          as_stream(stream));
-    note_launch(__func__);
-  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0); ct.fits) {
-    launch_softmax_nd_coltile<true, false>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, nullptr, nullptr,
-                                           false, as_stream(stream));
-    note_launch(__func__);
-  } else if (const bool vec = nd_vec(prefix_dim);
-             // (the kernel family, and with it the order of a pixel's sum, follows the shape alone, here as in the
-             // plain entry point)
-             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
-    hipStream_t s = as_stream(stream);
-    if (vec || (nd_overlapped_pairs(prefix_dim, dim0) && x != softmax)) {
-      launch_softmax_nd_reg<f32x4, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
-    } else {
-      launch_softmax_nd_reg<float, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s);
-    }
-    note_launch(__func__);
-  } else {
-    // shapes outside the register-resident kernel: the two passes, back to back
-    anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
-    anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
-  }
+  launch_softmax_nd_fused<false>(__func__, prefix_dim, dim0, dim1, x, cat_data, nullptr, softmax, nll, nullptr, cfg, stream);
 }
 
 // Additive: the same and the backward pass for a dy that is known before the forward pass (ones for a summed loss,
@@ -2766,43 +2851,22 @@ ANODE_EXPORT void anode_gpu_softmax_nd_cat_nll_fused_fwd_bwd_packed_f32(uint32_t
                                                                         const uint32_t *cat_data, const float *dy,
                                                                         float *softmax, float *nll, float *dx,
                                                                         const KernelConfig *cfg, CUstream_st *stream) {
-  const uint32_t len = checked_len(prefix_dim, dim0, dim1, __func__);
-  if (len == 0) return;
-  if (prefix_dim == 1) {  // the class axis is contiguous: the row form
-    launch_softmax_rows(__func__, dim0, dim1, x, softmax, stream, RowNll{cat_data, nll, false, dy, dx});
-  } else if (const SampleReg sr = nd_sample_reg(prefix_dim, dim0); sr.fits) {
-    launch_softmax_nd_samplereg<true, true>(sr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
-                                            as_stream(stream));
-    note_launch(__func__);
-  } else if (nd_tile_fits(prefix_dim, dim0)) {
-    launch_softmax_nd_tile<true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
-                                       as_stream(stream));
-    note_launch(__func__);
-  } else if (const ColReg cr = nd_col_reg(prefix_dim, dim0);
-             cr.fits && (nd_vec(prefix_dim) || (x != softmax && x != dx))) {
-    launch_softmax_nd_colreg<true, true>(cr, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
-                                         as_stream(stream));
-    note_launch(__func__);
-  } else if (const ColTile ct = nd_col_tile(prefix_dim, dim0);
-             ct.fits) {
-    launch_softmax_nd_coltile<true, true>(ct, prefix_dim, dim0, dim1, x, softmax, cat_data, nll, dy, dx, false,
-                                          as_stream(stream));
-    note_launch(__func__);
-  } else if (const bool vec = nd_vec(prefix_dim);
-             dim0 <= 32 || (vec && dim0 <= 256 && !nd_one_pixel_per_thread(prefix_dim, dim0, vec))) {
-    hipStream_t s = as_stream(stream);
-    if (vec || (nd_overlapped_pairs(prefix_dim, dim0) && x != softmax && x != dx)) {
-      launch_softmax_nd_reg<f32x4, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
-    } else {
-      launch_softmax_nd_reg<float, true, true>(prefix_dim, dim0, dim1, x, softmax, cat_data, nll, s, dy, dx);
-    }
-    note_launch(__func__);
-  } else {
-    // shapes outside the register-resident kernel: the three passes, back to back
-    anode_gpu_softmax_nd_packed_f32(prefix_dim, dim0, dim1, x, softmax, cfg, stream);
-    anode_gpu_softmax_nd_cat_nll_packed_f32(prefix_dim, dim0, dim1, softmax, cat_data, nll, cfg, stream);
-    anode_gpu_softmax_nd_cat_nll_bwd_packed_f32(prefix_dim, dim0, dim1, dy, softmax, cat_data, dx, cfg, stream);
+  launch_softmax_nd_fused<true>(__func__, prefix_dim, dim0, dim1, x, cat_data, dy, softmax, nll, dx, cfg, stream);
+}
+
+// Host-only view of nd_plan() for the tests: family, then the tiling of the family as 7 words (SampleReg: threads,
+// slots, G, PH; ColReg: 512, slots, Gt, PH, tiles per plane, xcd; ColTile: TP, L, tiles per plane).
+ANODE_EXPORT void anode_gpu_softmax_nd_plan_probe(uint32_t P, uint32_t C, int separate, uint32_t *out8) {
+  const NdPlan pl = nd_plan(P, C, separate != 0);
+  uint32_t v[8] = {uint32_t(pl.family), 0, 0, 0, 0, 0, 0, 0};
+  if (pl.family == NdFamily::SampleReg) {
+    v[1] = pl.sr.threads; v[2] = pl.sr.ns; v[3] = pl.sr.G; v[4] = pl.sr.PH;
+  } else if (pl.family == NdFamily::ColReg) {
+    v[1] = 512; v[2] = pl.cr.ns; v[3] = pl.cr.Gt; v[4] = pl.cr.PH; v[5] = pl.cr.tiles; v[6] = pl.cr.xcd;
+  } else if (pl.family == NdFamily::ColTile) {
+    v[1] = pl.ct.TP; v[2] = pl.ct.L; v[3] = pl.ct.tiles_per_sample;
   }
+  std::memcpy(out8, v, sizeof(v));
 }
 
 // Additive "ignore" variants (no counterpart in the reference, whose kernels give NaN and an unmasked gradient for

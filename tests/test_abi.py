@@ -470,3 +470,80 @@ def test_product_package_never_reaches_the_oracle():
                 assert "oracle" not in text.lower(), f"{os.path.join(dirpath, f)} mentions the oracle"
     needed = subprocess.run(["readelf", "-d", _lib.LIBRARY_PATH], capture_output=True, text=True).stdout
     assert "oracle" not in needed
+
+
+# ---- which kernel the channel-axis softmax takes for a shape (host logic of the library, no device call) ----
+
+ND_FAMILIES = {0: "rows", 1: "sample_reg", 2: "tile", 3: "col_reg", 4: "col_tile", 5: "pixel_per_thread", 6: "groups16",
+               7: "singles"}
+
+
+def _nd_plan(P, C, separate=True):
+    out = (ctypes.c_uint32 * 8)()
+    _lib.load().cdll.anode_gpu_softmax_nd_plan_probe(P, C, int(separate), out)
+    v = list(out)
+    return ND_FAMILIES[v[0]], v[1:]
+
+
+def test_softmax_nd_plan_invariants():
+    # Every tiling the planner hands out must hold the classes, fit the workgroup and cover the plane; a shape's
+    # family must not depend on whether the arrays are separate, except for planes that are not whole 16-byte groups
+    # (whose 16-byte kernels let the last two groups of a plane overlap and so need separate arrays).
+    shapes = [(P, C) for P in (1, 2, 4, 7, 8, 9, 16, 36, 49, 64, 100, 127, 128, 129, 132, 169, 196, 225, 256, 324, 400, 512,
+                               576, 784, 900, 1001, 1024, 1025, 1028, 2048, 4100, 4225, 16385, 65535, 65536, 131072, 263169,
+                               524288, 1 << 26)
+              for C in (1, 2, 3, 19, 21, 32, 33, 40, 64, 65, 100, 128, 129, 150, 200, 256, 257, 300, 400, 512, 513, 944,
+                        1000, 5000)]
+    seen = set()
+    for P, C in shapes:
+        fam, v = _nd_plan(P, C, True)
+        fam_alias, _ = _nd_plan(P, C, False)
+        seen.add(fam)
+        if P % 4 == 0 or fam in ("rows", "tile", "pixel_per_thread", "singles"):
+            assert fam_alias == fam, (P, C, fam, fam_alias)
+        else:
+            assert fam_alias in ("pixel_per_thread", "singles", "tile"), (P, C, fam, fam_alias)
+        if fam == "rows":
+            assert P == 1
+        elif fam == "sample_reg":
+            threads, ns, G, PH = v[:4]
+            assert P % 4 == 0 and G == P // 4 and threads in (256, 512, 1024) and ns in (8, 16), (P, C, v)
+            assert 1 <= PH <= 32 and G * PH <= threads and PH * ns >= C > 32, (P, C, v)
+        elif fam == "col_reg":
+            threads, ns, Gt, PH, tiles, xcd = v[:6]
+            P4 = -(-P // 4)
+            assert threads == 512 and ns in (8, 16) and P >= 128 and 33 <= C <= 512, (P, C, v)
+            assert 1 <= PH <= 32 and Gt * PH <= 512 and PH * ns >= C, (P, C, v)
+            assert Gt <= 64 and (tiles - 1) * Gt < P4 <= tiles * Gt, (P, C, v)
+            assert Gt == P4 or Gt % 4 == 0, (P, C, v)
+            assert xcd == (0 if P % 32 == 0 else 1), (P, C, v)
+        elif fam == "col_tile":
+            TP, L, tiles = v[:3]
+            assert P % 4 == 0 and TP % 4 == 0 and 16 <= TP <= 256 and L == 256 // TP >= 1, (P, C, v)
+            assert (tiles - 1) * TP < P <= tiles * TP and (C * TP + 5 * 256) * 4 <= 65536, (P, C, v)
+        elif fam == "groups16":
+            assert P % 4 == 0 or (P >= 8 and C <= 32), (P, C)
+        elif fam == "pixel_per_thread":
+            assert 33 <= C <= 128, (P, C)
+    assert seen == set(ND_FAMILIES.values()), seen
+
+
+def test_softmax_nd_plan_known_shapes():
+    # the shapes the measurements in the kernel comments were taken at
+    assert _nd_plan(524288, 19)[0] == "groups16"                      # config 3b: two lanes per pixel group
+    assert _nd_plan(196, 19)[0] == "tile" and _nd_plan(169, 19)[0] == "tile"
+    fam, v = _nd_plan(196, 100)
+    assert fam == "sample_reg" and v[:4] == [512, 16, 49, 10]
+    fam, v = _nd_plan(36, 256)
+    assert fam == "sample_reg" and v[:4] == [256, 16, 9, 28]
+    fam, v = _nd_plan(65536, 256)
+    assert fam == "col_reg" and v[:6] == [512, 16, 32, 16, 512, 0]
+    fam, v = _nd_plan(65536, 64)
+    assert fam == "col_reg" and v[:6] == [512, 8, 64, 8, 256, 0]
+    fam, v = _nd_plan(1024, 64)                                       # plane and sample powers of two: ragged runs
+    assert fam == "col_reg" and v[2:5] == [56, 9, 5]
+    fam, v = _nd_plan(900, 200)                                       # planes that are not whole lines: one XCD
+    assert fam == "col_reg" and v[1] == 8 and v[5] == 1
+    assert _nd_plan(4225, 21)[0] == "groups16" and _nd_plan(4225, 21, separate=False)[0] == "singles"
+    assert _nd_plan(4225, 150)[0] == "col_reg" and _nd_plan(4225, 150, separate=False)[0] != "col_reg"
+    assert _nd_plan(16, 944)[0] == "col_tile" and _nd_plan(65536, 1000)[0] == "groups16"
