@@ -2331,7 +2331,12 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P, 
 ColReg nd_col_reg(uint32_t P, uint32_t C) {
   ColReg cr = {0, 0, 0, 0, 0, false};
   if (tuning().nd_colreg == 0) return cr;
-  if (P < 128u || C <= 32u || C > 512u) return cr;
+  if (C <= 32u || C > 512u) return cr;
+  // Shorter planes keep the kernels tuned for them (whole samples in registers, the LDS tiles), except planes of 16
+  // pixels and more that are not whole 16-byte groups from 129 classes on, which none of those takes well:
+  // [49, 300] 1.6 -> 4.8 TB/s, [25, 512] 1.3 -> 5.3, [121, 150] 2.6 -> 5.1, [17, 200] 2.2 -> 5.4 (at 65 classes the
+  // LDS tiles are faster, 4.0-4.9 against 2.1-4.0, at 100 it depends on the plane).
+  if (P < 128u && (P % 4u == 0 || P < 16u || C < 129u)) return cr;
   const uint32_t P4 = (P + 3u) / 4u;  // (planes that are not whole 16-byte groups: the last group ends with the plane)
   const bool lines = P % 32u == 0;
   const uint32_t ns = (C <= 128u || (!lines && C <= 256u)) ? 8u : 16u;

@@ -512,7 +512,8 @@ def test_softmax_nd_plan_invariants():
         elif fam == "col_reg":
             threads, ns, Gt, PH, tiles, xcd = v[:6]
             P4 = -(-P // 4)
-            assert threads == 512 and ns in (8, 16) and P >= 128 and 33 <= C <= 512, (P, C, v)
+            assert threads == 512 and ns in (8, 16) and 33 <= C <= 512, (P, C, v)
+            assert P >= 128 or (P >= 16 and P % 4 != 0 and C >= 129), (P, C, v)
             assert 1 <= PH <= 32 and Gt * PH <= 512 and PH * ns >= C, (P, C, v)
             assert Gt <= 64 and (tiles - 1) * Gt < P4 <= tiles * Gt, (P, C, v)
             assert Gt == P4 or Gt % 4 == 0, (P, C, v)
@@ -547,3 +548,5 @@ def test_softmax_nd_plan_known_shapes():
     assert _nd_plan(4225, 21)[0] == "groups16" and _nd_plan(4225, 21, separate=False)[0] == "singles"
     assert _nd_plan(4225, 150)[0] == "col_reg" and _nd_plan(4225, 150, separate=False)[0] != "col_reg"
     assert _nd_plan(16, 944)[0] == "col_tile" and _nd_plan(65536, 1000)[0] == "groups16"
+    fam, v = _nd_plan(49, 300)                                        # short odd planes with many classes: whole planes
+    assert fam == "col_reg" and v[1:6] == [16, 13, 32, 1, 1]

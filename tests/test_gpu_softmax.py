@@ -272,7 +272,7 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # with the plane): two lanes per group up to 32 classes where no LDS tile holds the sample, column tiles
              # in registers from 129 pixels on
              (1001, 19, 2), (1023, 9, 2), (2049, 2, 3), (4225, 21, 1), (1026, 32, 2), (129, 33, 3), (131, 512, 1),
-             (4225, 64, 1), (1031, 300, 1),
+             (4225, 64, 1), (1031, 300, 1), (49, 300, 3), (17, 129, 5), (121, 200, 2), (25, 512, 2), (15, 300, 2),
              # the backward pass walked flat over planes that are not whole 16-byte groups (from 512 pixels on): the
              # shortest such plane and the next shorter one, an array whose last group is a partial one
              (513, 5, 3), (511, 5, 3), (515, 3, 1), (517, 1, 3),
