@@ -2212,7 +2212,7 @@ void launch_softmax_nd_samplereg(const SampleReg &sr, uint32_t P, uint32_t C, ui
   });
 }
 
-// Column tiles in registers, for 33 to 512 classes on planes of 128 pixels and more in whole 16-byte groups: the
+// Column tiles in registers, for 33 to 1024 classes on planes of 128 pixels and more: the
 // kernel above with a workgroup per run of Gt pixel groups of one sample instead of per sample.  Thread t =
 // phase * Gt + g holds pixel group g of the tile for the classes phase, phase + PH, ...: a wave reads, per slot, 64 / Gt
 // runs of Gt * 16 bytes, one per plane, and x is read once with nothing but the partial maxima and sums in LDS (the
@@ -2321,7 +2321,8 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P, 
 }
 
 // The tile a shape takes.  512 threads; 8 slots per thread up to 128 classes (256 on planes that are not whole
-// 128-byte lines), 16 beyond; runs of as many pixel groups as the threads then hold, up to 32 (64 up to 64 classes, 24
+// 128-byte lines), 16 up to 512, 32 beyond (some 170 registers: one workgroup per CU, which still reads x once where
+// the two-pass kernel reads it twice -- [1024, 1000] 3.0 -> 4.2 TB/s, [65536, 1000] 3.5 -> 4.4, [196, 800] 2.3 -> 3.7); runs of as many pixel groups as the threads then hold, up to 32 (64 up to 64 classes, 24
 // on planes that are not whole lines: [900, 100] 5.6 TB/s in runs of 24 groups, 5.4 in runs of 32), a multiple of 8
 // groups on planes of whole lines and of 4 otherwise, evened out over the tiles of a plane without adding a tile.
 // (Shorter runs that divide the plane exactly were slower where they fell under 16 groups: [324, 100] in runs of 12
@@ -2331,15 +2332,16 @@ __global__ __launch_bounds__(THREADS) void softmax_nd_colreg_kernel(uint32_t P, 
 ColReg nd_col_reg(uint32_t P, uint32_t C) {
   ColReg cr = {0, 0, 0, 0, 0, false};
   if (tuning().nd_colreg == 0) return cr;
-  if (C <= 32u || C > 512u) return cr;
+  if (C <= 32u || C > 1024u) return cr;
   // Shorter planes keep the kernels tuned for them (whole samples in registers, the LDS tiles), except planes of 16
   // pixels and more that are not whole 16-byte groups from 129 classes on, which none of those takes well:
   // [49, 300] 1.6 -> 4.8 TB/s, [25, 512] 1.3 -> 5.3, [121, 150] 2.6 -> 5.1, [17, 200] 2.2 -> 5.4 (at 65 classes the
-  // LDS tiles are faster, 4.0-4.9 against 2.1-4.0, at 100 it depends on the plane).
-  if (P < 128u && (P % 4u == 0 || P < 16u || C < 129u)) return cr;
+  // LDS tiles are faster, 4.0-4.9 against 2.1-4.0, at 100 it depends on the plane), and planes of whole groups from 513
+  // classes on, which no form of the sample kernel holds: [16, 1000] 3.0 -> 5.3, [64, 944] 3.1 -> 4.5.
+  if (P < 128u && ((P % 4u == 0 && C <= 512u) || P < 16u || C < 129u)) return cr;
   const uint32_t P4 = (P + 3u) / 4u;  // (planes that are not whole 16-byte groups: the last group ends with the plane)
   const bool lines = P % 32u == 0;
-  const uint32_t ns = (C <= 128u || (!lines && C <= 256u)) ? 8u : 16u;
+  const uint32_t ns = (C <= 128u || (!lines && C <= 256u)) ? 8u : (C <= 512u ? 16u : 32u);
   const uint32_t ph_need = (C + ns - 1u) / ns;  // at most 32
   const uint32_t step = lines ? 8u : 4u;
   uint32_t gt_max = 512u / ph_need;
@@ -2392,6 +2394,9 @@ void launch_softmax_nd_colreg(const ColReg &cr, uint32_t P, uint32_t C, uint32_t
     constexpr int NT = decltype(policy)::value;
     if (cr.ns == 8) {
       softmax_nd_colreg_kernel<8, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
+          P, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
+    } else if (cr.ns == 32) {
+      softmax_nd_colreg_kernel<32, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(
           P, C, cr.Gt, cr.PH, uint32_t(total), div_gt, div_tiles, ignore ? 1u : 0u, cr.xcd, x, y, cat, nll, dy, dx);
     } else {
       softmax_nd_colreg_kernel<16, 512, NLL, BWD, NT><<<blocks, launch_threads, 0, s>>>(

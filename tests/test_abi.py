@@ -493,7 +493,7 @@ def test_softmax_nd_plan_invariants():
                                576, 784, 900, 1001, 1024, 1025, 1028, 2048, 4100, 4225, 16385, 65535, 65536, 131072, 263169,
                                524288, 1 << 26)
               for C in (1, 2, 3, 19, 21, 32, 33, 40, 64, 65, 100, 128, 129, 150, 200, 256, 257, 300, 400, 512, 513, 944,
-                        1000, 5000)]
+                        1000, 1024, 1025, 5000)]
     seen = set()
     for P, C in shapes:
         fam, v = _nd_plan(P, C, True)
@@ -512,8 +512,8 @@ def test_softmax_nd_plan_invariants():
         elif fam == "col_reg":
             threads, ns, Gt, PH, tiles, xcd = v[:6]
             P4 = -(-P // 4)
-            assert threads == 512 and ns in (8, 16) and 33 <= C <= 512, (P, C, v)
-            assert P >= 128 or (P >= 16 and P % 4 != 0 and C >= 129), (P, C, v)
+            assert threads == 512 and ns in (8, 16, 32) and 33 <= C <= 1024, (P, C, v)
+            assert P >= 128 or (P >= 16 and C >= 129 and (P % 4 != 0 or C > 512)), (P, C, v)
             assert 1 <= PH <= 32 and Gt * PH <= 512 and PH * ns >= C, (P, C, v)
             assert Gt <= 64 and (tiles - 1) * Gt < P4 <= tiles * Gt, (P, C, v)
             assert Gt == P4 or Gt % 4 == 0, (P, C, v)
@@ -547,6 +547,9 @@ def test_softmax_nd_plan_known_shapes():
     assert fam == "col_reg" and v[1] == 8 and v[5] == 1
     assert _nd_plan(4225, 21)[0] == "groups16" and _nd_plan(4225, 21, separate=False)[0] == "singles"
     assert _nd_plan(4225, 150)[0] == "col_reg" and _nd_plan(4225, 150, separate=False)[0] != "col_reg"
-    assert _nd_plan(16, 944)[0] == "col_tile" and _nd_plan(65536, 1000)[0] == "groups16"
+    assert _nd_plan(16, 100)[0] == "col_tile" and _nd_plan(65536, 1025)[0] == "groups16"
+    assert _nd_plan(16, 944)[0] == "col_reg" and _nd_plan(16, 1025)[0] == "groups16"
+    fam, v = _nd_plan(65536, 1000)                                    # 513 to 1024 classes: 32 slots per thread
+    assert fam == "col_reg" and v[1:4] == [32, 16, 32]
     fam, v = _nd_plan(49, 300)                                        # short odd planes with many classes: whole planes
     assert fam == "col_reg" and v[1:6] == [16, 13, 32, 1, 1]

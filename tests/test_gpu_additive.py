@@ -206,7 +206,7 @@ def test_fused_batch_norm_equals_the_launch_sequence(oracle, S, C, N, masked):
                                    # column tiles in registers
                                    (128, 33, 3), (132, 512, 2), (900, 300, 1), (400, 200, 2), (2048, 257, 1), (4096, 64, 1),
                                    # planes that are not whole 16-byte groups through the 16-byte kernels
-                                   (1001, 19, 2), (2049, 2, 3), (4225, 21, 1), (129, 33, 3), (1031, 300, 1), (49, 300, 3), (17, 129, 5)])
+                                   (1001, 19, 2), (2049, 2, 3), (4225, 21, 1), (129, 33, 3), (1031, 300, 1), (49, 300, 3), (17, 129, 5), (196, 600, 2), (901, 700, 1)])
 def test_fused_softmax_nd_nll_equals_the_two_launches(oracle, P, C, N):
     g = np.random.default_rng(P + C)
     n = P * C * N

@@ -263,10 +263,11 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # column tiles over planes that are not whole 32-byte pieces (256 pixels and more, 65 to 128 classes,
              # too many pixel groups for a sample in registers), and one class more
              (676, 100, 1), (900, 65, 2), (1012, 128, 1), (900, 129, 1),
-             # column tiles in registers (33 to 512 classes, planes of 128 pixels and more in whole 16-byte groups):
-             # the fewest and the most classes and one more, the shortest plane and the next shorter one, 8 and 16
+             # column tiles in registers (33 to 1024 classes, planes of 128 pixels and more):
+             # the fewest and the most classes and one more, 32 slots per thread from 513 classes on, the shortest plane and the next shorter one, 8 and 16
              # slots per thread, ragged last tiles, planes that are and are not whole 128-byte lines
              (128, 33, 3), (124, 300, 2), (132, 512, 2), (1028, 513, 1), (900, 300, 1), (400, 200, 2), (4100, 40, 1),
+             (196, 600, 2), (1024, 1024, 1), (1028, 1025, 1), (901, 700, 1), (16, 1024, 2), (64, 600, 2), (100, 513, 1),
              (2048, 257, 1), (1024, 512, 1), (324, 256, 2), (4096, 64, 1),
              # planes that are not whole 16-byte groups through the 16-byte kernels (the last group of a plane ends
              # with the plane): two lanes per group up to 32 classes where no LDS tile holds the sample, column tiles
