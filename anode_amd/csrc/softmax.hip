@@ -2596,7 +2596,7 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_kernel(uin
 // the array.  A group inside one plane fetches dy and labels with 16-byte accesses at 4-byte-aligned addresses; the
 // one group per plane that lies across its end, and the array's last group, go element by element.  The stores stay
 // aligned 16-byte ones, which the kernels with one pixel per thread do not have: [4225, 19] 4.3 -> 5.0 TB/s,
-// [1025, 100] 3.2 -> 5.1, [961, 64] 4.0 -> 5.1, [65535, 4] 4.2 -> 5.1.
+// [1025, 100] 3.2 -> 5.1, [961, 64] 4.0 -> 5.2, [65535, 4] 4.2 -> 5.1.
 template <bool ACC, int NT>
 __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_any_kernel(uint32_t P, uint32_t C, uint32_t len,
                                                                                  FastDiv div_p, FastDiv div_c,
@@ -2629,17 +2629,39 @@ __global__ __launch_bounds__(kBlock) void softmax_nd_cat_nll_bwd_flat_any_kernel
       }
       store_stream<NT>(reinterpret_cast<f32x4 *>(dx + e), out);
     } else {
-      for (uint32_t w = 0; w < 4u && uint64_t(e) + w < len; ++w) {
-        uint32_t pl, rr;
-        div_p.divmod(e + w, pl, rr);
-        const uint32_t n = div_c.div(pl);
-        const uint32_t k = pl - n * C;
-        const size_t pix = size_t(n) * P + rr;
-        const uint32_t label = cat[pix];
-        float d = dy[pix];
-        if (ignore && label >= C) d = 0.0f;
-        const float t = prob[e + w] - float(label == k);
-        dx[e + w] = ACC ? fmaf(d, t, dx[e + w]) : d * t;
+      // The group lies across the end of a plane (P >= 16: of one plane only) or of the array.  Its elements' planes
+      // and pixels follow from the first one's; everything is requested before anything is used.
+      uint32_t kk[4], label[4];
+      size_t pix[4];
+      float d[4], pr[4], old[4];
+      bool in[4];
+      const uint32_t n0 = div_c.div(plane);
+      const uint32_t k0 = plane - n0 * C;
+#pragma unroll
+      for (uint32_t w = 0; w < 4u; ++w) {
+        in[w] = uint64_t(e) + w < len;
+        const bool next = r + w >= P;            // the element belongs to the next plane
+        const uint32_t rr = next ? r + w - P : r + w;
+        uint32_t k = next ? k0 + 1u : k0, n = n0;
+        if (k == C) {                            // ... which is the first plane of the next sample
+          k = 0u;
+          n += 1u;
+        }
+        kk[w] = k;
+        pix[w] = size_t(n) * P + rr;
+      }
+#pragma unroll
+      for (uint32_t w = 0; w < 4u; ++w) {
+        label[w] = in[w] ? cat[pix[w]] : 0u;
+        d[w] = in[w] ? dy[pix[w]] : 0.0f;
+        pr[w] = in[w] ? prob[e + w] : 0.0f;
+        old[w] = (ACC && in[w]) ? dx[e + w] : 0.0f;
+      }
+#pragma unroll
+      for (uint32_t w = 0; w < 4u; ++w) {
+        if (ignore && label[w] >= C) d[w] = 0.0f;
+        const float t = pr[w] - float(label[w] == kk[w]);
+        if (in[w]) dx[e + w] = ACC ? fmaf(d[w], t, old[w]) : d[w] * t;
       }
     }
   }
@@ -2680,9 +2702,11 @@ void launch_softmax_nd_cat_nll_bwd(const char *symbol, uint32_t P, uint32_t C, u
           <<<stream_grid(total_groups, 1), kBlock, 0, s>>>(P, C, total_groups, div_gpp, div_c, ignore ? 1u : 0u, dy, prob,
                                                           cat, dx);
     });
-  } else if (!vec && P >= 512 && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
-    // (shorter planes: a wave of 256 elements then always holds a group that lies across the end of a plane and
-    // walks it element by element, [169, 19] accumulating 4.7 TB/s with one pixel per thread against 3.4 here)
+  } else if (!vec && P >= (ACC ? 200u : 64u) && P <= uint32_t(tuning().nd_bwd_flat_max_plane)) {
+    // (shorter planes: every wave of 256 elements then holds groups that lie across the end of a plane and go
+    // element by element.  One pixel per thread is faster below 64 pixels, [33, 19] 3.8 TB/s against 2.7, and when
+    // accumulating below some 200, [129, 19] 4.7 against 4.3; above, [361, 19] 4.0 -> 4.7 and accumulating 4.7 -> 5.0,
+    // [129, 100] 3.1 -> 4.7.)
     const FastDiv div_p(P), div_c(C);
     with_stream_policy(policy_for_outputs(stream_policy(size_t(len) * sizeof(float), tuning().nontemporal), dx), [&](auto policy) {
       softmax_nd_cat_nll_bwd_flat_any_kernel<ACC, decltype(policy)::value>

@@ -274,9 +274,9 @@ ND_SHAPES = [(64, 19, 2), (4, 3, 5), (5, 3, 4), (1, 10, 6), (2048, 19, 2), (100,
              # in registers from 129 pixels on
              (1001, 19, 2), (1023, 9, 2), (2049, 2, 3), (4225, 21, 1), (1026, 32, 2), (129, 33, 3), (131, 512, 1),
              (4225, 64, 1), (1031, 300, 1), (49, 300, 3), (17, 129, 5), (121, 200, 2), (25, 512, 2), (15, 300, 2),
-             # the backward pass walked flat over planes that are not whole 16-byte groups (from 512 pixels on): the
-             # shortest such plane and the next shorter one, an array whose last group is a partial one
-             (513, 5, 3), (511, 5, 3), (515, 3, 1), (517, 1, 3),
+             # the backward pass walked flat over planes that are not whole 16-byte groups (from 64 pixels on, from 200
+             # when accumulating): the shortest such planes and the next shorter ones, arrays whose last group is partial
+             (513, 5, 3), (511, 5, 3), (515, 3, 1), (517, 1, 3), (65, 5, 7), (63, 5, 7), (201, 3, 5), (199, 3, 5),
              # planes of more than 131072 pixels: the backward pass gives a thread four pixels and walks their classes
              (131076, 5, 1), (131080, 19, 1), (131073, 3, 1)]
 
