@@ -169,7 +169,12 @@ def test_upcast(oracle):
 
 # ---- one-hot -------------------------------------------------------------------
 
-@pytest.mark.parametrize("d0,K,d2", [(1, 4, 7), (5, 3, 2), (64, 19, 3), (100, 1, 2), (7, 10, 5), (4096, 5, 2), (12, 40, 3)])
+@pytest.mark.parametrize("d0,K,d2", [(1, 4, 7), (5, 3, 2), (64, 19, 3), (100, 1, 2), (7, 10, 5), (4096, 5, 2), (12, 40, 3),
+                                     # the flat walk (planes of whole 16-byte groups from 16 pixels on, any plane from 512
+                                     # on): its shortest planes and the next shorter ones, groups across the end of a
+                                     # plane, of a sample and of the array, one class
+                                     (16, 3, 5), (20, 7, 3), (512, 3, 2), (513, 5, 3), (511, 5, 3), (515, 3, 1), (517, 1, 3),
+                                     (1025, 19, 2), (4225, 2, 1)])
 def test_one_hot(oracle, d0, K, d2):
     g = np.random.default_rng(d0 + K)
     lab = g.integers(0, K + 2, d0 * d2).astype(np.uint32)  # some labels have no class: all-zero column
