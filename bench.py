@@ -73,8 +73,8 @@ MEASURED_TRAFFIC = {
     ("anode_gpu_batch_var_bwd_3d1_packed_accumulate_f32", "bn_bwd_cfg2b"): (308434067, "bn_maps"),
     ("anode_gpu_positive_clip_flat_map_bwd_f32", "relu_cfg4"): (1610547205, "flat_maps"),
     ("anode_gpu_softmax_nd_packed_f32", "softmax_cfg3b"): (637597563, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291489265, "softmax"),
-    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671292527, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_packed_f32", "softmax_cfg3b"): (291407352, "softmax"),
+    ("anode_gpu_softmax_nd_cat_nll_bwd_packed_f32", "softmax_cfg3b"): (671288431, "softmax"),
     ("anode_gpu_dequantize_u8_packed_f32", "cast_cfg1"): (192699228, "flat_maps"),
     ("anode_gpu_upcast_u8_packed_u32", "cast_cfg1"): (192703324, "flat_maps"),
 }
@@ -92,7 +92,7 @@ TRAFFIC_FAMILY_FINGERPRINT = {
     "bn_maps": "9d94a1d3c0e0f479",
     "bn_reductions": "e27eb3a6158f909f",
     "flat_maps": "c8b36a639e6d43e9",
-    "softmax": "866bdce3d866285c",
+    "softmax": "a3e766a866176ae6",
 }
 
 
